@@ -1,0 +1,204 @@
+/*
+ * mfsdp_hip.h -- C ABI of libmfsdp_hip.so: MatrixFSDP's per-rank copy-in /
+ * copy-out path and owner-rank optimizer update as hand-written gfx950 (CDNA4)
+ * HIP kernels.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes; device pointers are raw HBM addresses on the
+ *     current HIP device; `stream` is a hipStream_t passed as void* (NULL = the
+ *     default stream);
+ *   - every call validates its arguments on the host, enqueues its kernels on
+ *     `stream` and returns without synchronising; tensors are borrowed for the
+ *     duration of the enqueued work;
+ *   - return value 0 = success; any other value is an error code and
+ *     mfsdp_last_error() holds a message for the calling thread.  A binding
+ *     turns non-zero into the host language's exception (the reference's
+ *     TORCH_CHECK -> RuntimeError convention, matrix_copy.cpp:60-78, 86-94);
+ *   - only the *_create / *_destroy calls allocate or free device memory.
+ *
+ * Element offsets, not bytes, everywhere; `elem_bytes` in {1, 2, 4, 8}.
+ */
+#ifndef MFSDP_HIP_H_
+#define MFSDP_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MFSDP_OK 0
+#define MFSDP_ERR_INVALID 1   /* bad argument (null pointer, negative size, out of range, misaligned) */
+#define MFSDP_ERR_HIP 2       /* a HIP runtime call failed */
+#define MFSDP_ERR_UNSUPPORTED 3
+
+/* dtype codes used by the cast / optimizer entry points */
+#define MFSDP_F32 0
+#define MFSDP_BF16 1
+
+/* conversion a segment program applies while copying */
+#define MFSDP_CONVERT_NONE 0         /* raw element move, any elem_bytes */
+#define MFSDP_CONVERT_BF16_TO_F32 1  /* exact widening (Tensor.to(float32)) */
+#define MFSDP_CONVERT_F32_TO_BF16 2  /* round-to-nearest-even, NaN -> 0x7FC0 (Tensor.to(bfloat16)) */
+
+const char* mfsdp_last_error(void);
+/* ABI version of the library; bumped on any signature change. */
+int mfsdp_abi_version(void);
+
+/* ------------------------------------------------------------------ copy */
+
+/*
+ * out[o] = in[input_offset + o] for o < out_numel.
+ * Replaces copy_range (matrix_fsdp/kernels/native/matrix_copy.cpp:85-99,
+ * matrix_copy_cuda.cu:25-36, 69-87).  Errors as the reference: negative
+ * offset, range exceeding the input.  out_numel == 0 returns at once.
+ */
+int mfsdp_copy_range(const void* in, int64_t in_numel, void* out, int64_t out_numel,
+                     int64_t input_offset, int elem_bytes, void* stream);
+
+/*
+ * out[global_starts[s] + o] = local[local_starts[s] + o] for o < numels[s].
+ * Replaces copy_rank_segments_to_full (matrix_copy.cpp:53-83,
+ * matrix_copy_cuda.cu:8-23, 38-67).  The three metadata arrays are HOST arrays
+ * of n_segments int64 each (the reference passes device tensors it caches per
+ * layout, kernels/native.py:470-489; here the cached object is the segment
+ * program below, and this call is the uncached convenience form: it builds a
+ * throw-away program, so it allocates and synchronises -- use a program on hot
+ * paths).  n_segments == 0 returns at once.
+ */
+int mfsdp_copy_rank_segments_to_full(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                                     const int64_t* global_starts, const int64_t* local_starts,
+                                     const int64_t* numels, int64_t n_segments, int elem_bytes, void* stream);
+
+/*
+ * Segment program: a layout's whole copy (every rank, every segment, pad
+ * zero-fill, optional dtype conversion) compiled once into device-resident
+ * tables and replayed with ONE kernel launch per buffer.
+ *
+ * A run is a 2-D strided block, in elements:
+ *     for r < rows, c < row_len:
+ *         dst[dst_off + r*dst_stride + c] = convert(src[src_id][src_off + r*src_stride + c])
+ * src_id = -1 writes zeros instead (pad tails: new_zeros / packed.zero_() in
+ * matrix_fsdp/runtime/collectives.py:236-237 and runtime/grad_bucket.py:106).
+ * A plain segment is a run with rows = 1.  It covers
+ *   pack    _pack_full_tensor_by_rank_segments  (runtime/flat_buffer.py:1304-1316) fused with the
+ *           zero-padded all-gather staging       (runtime/collectives.py:236-237, 248-249),
+ *   unpack  un-pad                               (runtime/collectives.py:264-272) fused with
+ *           _unpack_rank_shards_to_full_tensor   (runtime/flat_buffer.py:1318-1333),
+ *   owner self-copy _copy_local_rank_segments    (runtime/collectives.py:495-503),
+ *   grad copy-in    fill_reduce_scatter_input    (runtime/grad_bucket.py:71-116, 200-225),
+ *                   compact owner fill           (runtime/flat_buffer.py:1232-1252),
+ *   with the dtype casts of runtime/flat_buffer.py:1186-1206 folded in.
+ * Destination runs of one program must not overlap each other.
+ */
+typedef struct mfsdp_copy_run {
+  int64_t src_off;
+  int64_t dst_off;
+  int64_t row_len;
+  int64_t rows;
+  int64_t src_stride;
+  int64_t dst_stride;
+  int32_t src_id;   /* index into the srcs[] array given at run time; -1 = zero fill */
+  int32_t reserved;
+} mfsdp_copy_run;
+
+typedef struct mfsdp_segment_program mfsdp_segment_program;
+
+/*
+ * Merges consecutive segments with equal length and constant source /
+ * destination pitch into 2-D runs (a 2x2 block shard of an R x C matrix: R/2
+ * row segments -> one run).  `segs` holds n_segs plain runs (rows == 1);
+ * `out` has room for n_segs runs; returns the number written (host only).
+ */
+int64_t mfsdp_merge_segment_runs(const mfsdp_copy_run* segs, int64_t n_segs, mfsdp_copy_run* out);
+
+/*
+ * Validates the runs against the extents (src_numels[n_srcs], dst_numel),
+ * compiles and uploads them.  Allocates device memory; synchronous.
+ * `convert` is one of MFSDP_CONVERT_*; elem_bytes is the element size for
+ * MFSDP_CONVERT_NONE (ignored otherwise: 2 -> 4 or 4 -> 2 bytes).
+ */
+int mfsdp_segment_program_create(const mfsdp_copy_run* runs, int64_t n_runs,
+                                 const int64_t* src_numels, int32_t n_srcs, int64_t dst_numel,
+                                 int convert, int elem_bytes, mfsdp_segment_program** out);
+void mfsdp_segment_program_destroy(mfsdp_segment_program* program);
+/* Algorithmic bytes one run of the program moves: bytes read + bytes written (zero fill counts as written). */
+int64_t mfsdp_segment_program_bytes(const mfsdp_segment_program* program);
+int64_t mfsdp_segment_program_num_runs(const mfsdp_segment_program* program);
+
+/*
+ * Replays the program: srcs[i] is the device base of source i and must hold
+ * at least the src_numels[i] elements given at create time, dst at least
+ * dst_numel.  One kernel launch, no allocation, no synchronisation (the first
+ * call with base pointers less aligned than any earlier call compiles a
+ * narrower-vector variant of the tables; that one call allocates).
+ */
+int mfsdp_segment_program_run(mfsdp_segment_program* program, const void* const* srcs, int32_t n_srcs,
+                              void* dst, void* stream);
+
+/* Launch tuning for experiments: blocks per CU of the persistent copy grid
+ * (0 = library default), non-temporal load/store hints (0/1, -1 = default) and
+ * 128-bit loads in flight per lane (4 or 8; applies to programs created afterwards). */
+void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll);
+
+/* ------------------------------------------------------------------ cast */
+
+/*
+ * dst = convert(src) element-wise over `numel` contiguous elements: the
+ * Tensor.to(dtype) of _maybe_to_param_dtype / _maybe_to_reduce_dtype /
+ * _maybe_to_local_dtype (matrix_fsdp/runtime/flat_buffer.py:1186-1206).
+ */
+int mfsdp_cast(const void* src, void* dst, int64_t numel, int convert, void* stream);
+
+/* ------------------------------------------------------------------ Muon */
+
+/*
+ * Bytes of device workspace mfsdp_muon_step / mfsdp_newton_schulz need for an
+ * rows x cols matrix (0 on invalid shape).
+ */
+int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols);
+
+/*
+ * Quintic Newton-Schulz orthogonalisation of one matrix, the arithmetic of
+ * torch.optim._muon._zeropower_via_newtonschulz (torch/optim/_muon.py:31-70)
+ * that MixedMuonAdamWOptimizer.step reaches through torch.optim.Muon
+ * (matrix_fsdp/optim/wrapper.py:497-516): bf16 operands, fp32 accumulation,
+ * every product rounded to bf16, Frobenius normalisation with max(norm, eps).
+ * `update` is rows x cols row-major of dtype `update_dtype` (MFSDP_F32 or
+ * MFSDP_BF16); `out` is rows x cols bf16.
+ */
+int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t rows, int64_t cols,
+                        float a, float b, float c, int steps, float eps,
+                        void* out_bf16, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * One matrix of torch.optim._muon._single_tensor_muon (torch/optim/_muon.py:285-318):
+ *   buf <- buf + (1-momentum)*(grad - buf);  U = nesterov ? grad + momentum*(buf - grad) : buf
+ *   O = NewtonSchulz(U);  param <- param*(1 - lr*weight_decay) - adjusted_lr*O
+ * param / grad / momentum buffer share one dtype (`dtype`), as the reference's
+ * local shard, local grad shard and zeros_like(grad) state do
+ * (matrix_fsdp/runtime/flat_buffer.py:790-803).  adjusted_lr is the caller's
+ * _adjust_lr(lr, fn, shape) (torch/optim/_muon.py:73-84).
+ */
+int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols,
+                    float lr, float weight_decay, float momentum, int nesterov,
+                    float a, float b, float c, int steps, float eps, float adjusted_lr,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ AdamW */
+
+/*
+ * Fused single-launch AdamW over a flat fp32 shard (the arithmetic of
+ * torch/optim/adam.py:347-547 with decoupled weight decay, reached through
+ * matrix_fsdp/optim/wrapper.py:439, 497-516; state laid out flat as in
+ * matrix_fsdp/optim/adamw_state.py:177-218).  `step` is the 1-based step
+ * count after this update.  grad_dtype: MFSDP_F32 or MFSDP_BF16.
+ */
+int mfsdp_adamw_step(float* param, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
+                     int64_t numel, int64_t step, float lr, float beta1, float beta2, float eps,
+                     float weight_decay, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MFSDP_HIP_H_ */

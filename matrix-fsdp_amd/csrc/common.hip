@@ -1,0 +1,35 @@
+// Error string, ABI version and device queries of libmfsdp_hip.
+#include "mfsdp_common.h"
+
+#include <mutex>
+
+namespace mfsdp {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int device_cu_count() {
+  static std::mutex mu;
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev] = cus;
+  }
+  return cached[dev];
+}
+
+}  // namespace mfsdp
+
+extern "C" const char* mfsdp_last_error(void) { return mfsdp::g_last_error; }
+extern "C" int mfsdp_abi_version(void) { return 1; }
