@@ -1,0 +1,215 @@
+// Element-wise stages of the owner-rank Muon update (everything around the Newton-Schulz GEMMs):
+//   1. momentum + Nesterov + bf16 rounding + partial sums of squares,
+//   2. Frobenius norm (rounded to bf16 and clamped, as the bf16 tensor ops of the reference do),
+//   3. division by the norm, written both as X (short side first) and X^T into zero-padded buffers,
+//   4. the parameter update  p <- p*(1 - lr*wd) - adjusted_lr * O.
+// All are HBM-bound and small next to the GEMMs.
+#include "muon_elementwise.h"
+
+#include "mfsdp_common.h"
+
+#include <algorithm>
+
+namespace mfsdp {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
+
+// round to nearest even; inputs here are finite
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+  return static_cast<uint16_t>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// Tensor.lerp as ATen evaluates it.
+__device__ __forceinline__ float lerp_aten(float start, float end, float weight) {
+  const float diff = end - start;
+  return weight < 0.5f ? start + weight * diff : end - diff * (1.0f - weight);
+}
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+  static __device__ __forceinline__ float load(const float* p, int64_t i) { return p[i]; }
+  static __device__ __forceinline__ void store(float* p, int64_t i, float v) { p[i] = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <>
+struct Elem<uint16_t> {  // bf16 storage
+  static __device__ __forceinline__ float load(const uint16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+  static __device__ __forceinline__ void store(uint16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+  static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  float total = 0.0f;
+  if (threadIdx.x == 0) {
+    for (int w = 0; w < kThreads / 64; ++w) total += lds[w];
+  }
+  return total;  // valid in thread 0
+}
+
+// MOMENTUM: buf <- lerp(buf, g, 1-mu); u = nesterov ? lerp(g, buf, mu) : buf.   !MOMENTUM: u = g.
+// xraw <- bf16(u); partials[block] = sum of bf16(u)^2 over the block's elements.
+template <typename T, bool MOMENTUM>
+__global__ void __launch_bounds__(kThreads)
+momentum_kernel(const T* __restrict__ grad, T* __restrict__ buf, uint16_t* __restrict__ xraw, float* __restrict__ partials,
+                int64_t numel, float momentum, float one_minus_momentum, int nesterov) {
+  __shared__ float lds[kThreads / 64];
+  float sumsq = 0.0f;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < numel; i += stride) {
+    const float g = Elem<T>::load(grad, i);
+    float u = g;
+    if constexpr (MOMENTUM) {
+      const float b = Elem<T>::round(lerp_aten(Elem<T>::load(buf, i), g, one_minus_momentum));
+      Elem<T>::store(buf, i, b);
+      u = nesterov ? Elem<T>::round(lerp_aten(g, b, momentum)) : b;
+    }
+    const uint16_t xb = f32_to_bf16(u);
+    xraw[i] = xb;
+    const float xf = bf16_to_f32(xb);
+    sumsq += xf * xf;
+  }
+  const float total = block_sum(sumsq, lds);
+  if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
+// scalars[0] = max(bf16(sqrt(sum partials)), bf16(eps))
+__global__ void __launch_bounds__(kThreads)
+norm_kernel(const float* __restrict__ partials, int n_partials, float eps, float* __restrict__ scalars) {
+  __shared__ double lds[kThreads];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n_partials; i += kThreads) s += static_cast<double>(partials[i]);
+  lds[threadIdx.x] = s;
+  __syncthreads();
+  for (int off = kThreads / 2; off > 0; off >>= 1) {
+    if (static_cast<int>(threadIdx.x) < off) lds[threadIdx.x] += lds[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float norm = bf16_to_f32(f32_to_bf16(__fsqrt_rn(static_cast<float>(lds[0]))));
+    const float floor_ = bf16_to_f32(f32_to_bf16(eps));
+    scalars[0] = norm > floor_ ? norm : floor_;
+  }
+}
+
+// 64 x 64 tile of the zero-padded outputs per block:
+//   same [r][c]  = bf16(x[r][c] / norm)   (rows_pad x cols_pad, ld = cols_pad)
+//   trans[c][r]  = same[r][c]             (cols_pad x rows_pad, ld = rows_pad)
+// with x = 0 outside rows x cols.
+__global__ void __launch_bounds__(kThreads)
+scale_transpose_kernel(const uint16_t* __restrict__ xraw, int rows, int cols, const float* __restrict__ scalars,
+                       uint16_t* __restrict__ same, uint16_t* __restrict__ trans, int rows_pad, int cols_pad) {
+  __shared__ uint16_t tile[64][66];
+  const float norm = scalars[0];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
+    const int lr = e >> 6, lc = e & 63;
+    const int r = r0 + lr, c = c0 + lc;
+    uint16_t v = 0;
+    if (r < rows && c < cols) v = f32_to_bf16(__fdiv_rn(bf16_to_f32(xraw[static_cast<int64_t>(r) * cols + c]), norm));
+    tile[lr][lc] = v;
+    same[static_cast<int64_t>(r) * cols_pad + c] = v;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
+    const int lc = e >> 6, lr = e & 63;  // consecutive threads walk down a column of the tile = along a row of trans
+    trans[static_cast<int64_t>(c0 + lc) * rows_pad + r0 + lr] = tile[lr][lc];
+  }
+}
+
+// p <- round(round(p * decay) + neg_lr * o) over rows x cols, o read with leading dimension ldo.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+apply_kernel(T* __restrict__ param, const uint16_t* __restrict__ ortho, int rows, int cols, int ldo, float decay, float neg_lr) {
+  for (int r = blockIdx.y; r < rows; r += gridDim.y) {
+    for (int c = blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads) {
+      const int64_t i = static_cast<int64_t>(r) * cols + c;
+      const float p = Elem<T>::round(Elem<T>::load(param, i) * decay);
+      Elem<T>::store(param, i, p + neg_lr * bf16_to_f32(ortho[static_cast<int64_t>(r) * ldo + c]));
+    }
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+extract_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ ortho, int rows, int cols, int ldo) {
+  for (int r = blockIdx.y; r < rows; r += gridDim.y)
+    for (int c = blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads)
+      out[static_cast<int64_t>(r) * cols + c] = ortho[static_cast<int64_t>(r) * ldo + c];
+}
+
+int partial_blocks(int64_t numel) {
+  const int64_t want = (numel + kThreads * 8 - 1) / (kThreads * 8);
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(want, kMuonMaxPartials)));
+}
+
+}  // namespace
+
+int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, float momentum, int nesterov, bool with_momentum,
+                  void* xraw, float* partials, int* n_partials, hipStream_t stream) {
+  const int blocks = partial_blocks(numel);
+  *n_partials = blocks;
+  // the scalar the reference hands to lerp_ is the Python double 1 - momentum
+  const float one_minus = static_cast<float>(1.0 - static_cast<double>(momentum));
+  auto x = static_cast<uint16_t*>(xraw);
+  if (dtype == MFSDP_F32) {
+    auto g = static_cast<const float*>(grad);
+    auto b = static_cast<float*>(buf);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<float, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<float, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+  } else {
+    auto g = static_cast<const uint16_t*>(grad);
+    auto b = static_cast<uint16_t*>(buf);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<uint16_t, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<uint16_t, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+  }
+  MFSDP_CHECK_LAUNCH("momentum_kernel");
+  return MFSDP_OK;
+}
+
+int muon_norm(const float* partials, int n_partials, float eps, float* scalars, hipStream_t stream) {
+  hipLaunchKernelGGL(norm_kernel, dim3(1), dim3(kThreads), 0, stream, partials, n_partials, eps, scalars);
+  MFSDP_CHECK_LAUNCH("norm_kernel");
+  return MFSDP_OK;
+}
+
+int muon_scale_transpose(const void* xraw, int rows, int cols, const float* scalars, void* same, void* trans, int rows_pad,
+                         int cols_pad, hipStream_t stream) {
+  const dim3 grid(cols_pad / 64, rows_pad / 64);
+  hipLaunchKernelGGL(scale_transpose_kernel, grid, dim3(kThreads), 0, stream, static_cast<const uint16_t*>(xraw), rows, cols,
+                     scalars, static_cast<uint16_t*>(same), static_cast<uint16_t*>(trans), rows_pad, cols_pad);
+  MFSDP_CHECK_LAUNCH("scale_transpose_kernel");
+  return MFSDP_OK;
+}
+
+int muon_apply(void* param, int dtype, const void* ortho, int rows, int cols, int ldo, float decay, float neg_lr,
+               hipStream_t stream) {
+  const dim3 grid(std::max(1, std::min((cols + kThreads - 1) / kThreads, 64)), std::min(rows, 65535));
+  auto o = static_cast<const uint16_t*>(ortho);
+  if (dtype == MFSDP_F32)
+    hipLaunchKernelGGL((apply_kernel<float>), grid, dim3(kThreads), 0, stream, static_cast<float*>(param), o, rows, cols, ldo, decay, neg_lr);
+  else
+    hipLaunchKernelGGL((apply_kernel<uint16_t>), grid, dim3(kThreads), 0, stream, static_cast<uint16_t*>(param), o, rows, cols, ldo, decay, neg_lr);
+  MFSDP_CHECK_LAUNCH("apply_kernel");
+  return MFSDP_OK;
+}
+
+int muon_extract(void* out, const void* ortho, int rows, int cols, int ldo, hipStream_t stream) {
+  const dim3 grid(std::max(1, std::min((cols + kThreads - 1) / kThreads, 64)), std::min(rows, 65535));
+  hipLaunchKernelGGL(extract_kernel, grid, dim3(kThreads), 0, stream, static_cast<uint16_t*>(out),
+                     static_cast<const uint16_t*>(ortho), rows, cols, ldo);
+  MFSDP_CHECK_LAUNCH("extract_kernel");
+  return MFSDP_OK;
+}
+
+}  // namespace mfsdp

@@ -1,0 +1,118 @@
+"""``FusedAdamW``: AdamW on the HIP kernel, one launch per contiguous run of parameters.
+
+Hyper-parameters, parameter-group keys and state keys (``step``, ``exp_avg``,
+``exp_avg_sq``) are those of ``torch.optim.AdamW``, the optimizer the reference
+builds for everything Muon does not take (matrix_fsdp/optim/wrapper.py:431-439);
+the arithmetic is the single-tensor path of torch/optim/adam.py:347-547.  When
+the parameters are views of one flat shard, their grads views of one local
+grad shard and their moments views of flat state buffers
+(``initialize_flat_adamw_state``), neighbouring parameters are merged and the
+whole shard is updated by a single launch.
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+from torch.optim.optimizer import Optimizer
+
+from . import functional as F
+
+
+class FusedAdamW(Optimizer):
+    def __init__(
+        self,
+        params,
+        lr: float = 1e-3,
+        betas: tuple[float, float] = (0.9, 0.999),
+        eps: float = 1e-8,
+        weight_decay: float = 1e-2,
+        amsgrad: bool = False,
+        *,
+        maximize: bool = False,
+    ) -> None:
+        if isinstance(lr, Tensor):
+            raise ValueError("FusedAdamW takes a float lr")
+        if not 0.0 <= lr:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon value: {eps}")
+        if not 0.0 <= betas[0] < 1.0:
+            raise ValueError(f"Invalid beta parameter at index 0: {betas[0]}")
+        if not 0.0 <= betas[1] < 1.0:
+            raise ValueError(f"Invalid beta parameter at index 1: {betas[1]}")
+        if not 0.0 <= weight_decay:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        if amsgrad or maximize:
+            raise NotImplementedError("FusedAdamW supports neither amsgrad nor maximize")
+        defaults = {"lr": lr, "betas": betas, "eps": eps, "weight_decay": weight_decay, "amsgrad": False, "maximize": False}
+        super().__init__(params, defaults)
+
+    def _init_state(self, p: Tensor) -> dict:
+        state = self.state[p]
+        if len(state) == 0:
+            state["step"] = torch.tensor(0.0, dtype=torch.float32)
+            state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+        return state
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for group in self.param_groups:
+            entries = []
+            for p in group["params"]:
+                if p.grad is None or p.numel() == 0:
+                    continue
+                if p.grad.is_sparse:
+                    raise RuntimeError("AdamW does not support sparse gradients")
+                if p.dtype != torch.float32:
+                    raise RuntimeError(f"FusedAdamW updates float32 parameters, got {p.dtype}")
+                state = self._init_state(p)
+                state["step"] += 1
+                entries.append((p.data, p.grad.contiguous(), state["exp_avg"], state["exp_avg_sq"], int(state["step"].item())))
+            for param, grad, exp_avg, exp_avg_sq, step in _merge_contiguous(entries):
+                F.adamw_step(
+                    param, grad, exp_avg, exp_avg_sq, step,
+                    lr=group["lr"], betas=group["betas"], eps=group["eps"], weight_decay=group["weight_decay"],
+                )
+        return loss
+
+
+def _follows(prev: Tensor, nxt: Tensor) -> bool:
+    return (
+        prev.dtype == nxt.dtype
+        and prev.device == nxt.device
+        and prev.is_contiguous()
+        and nxt.is_contiguous()
+        and prev.untyped_storage().data_ptr() == nxt.untyped_storage().data_ptr()
+        and prev.data_ptr() + prev.numel() * prev.element_size() == nxt.data_ptr()
+    )
+
+
+def _merge_contiguous(entries):
+    """Merges neighbours whose parameter, grad and both moments each continue
+    the previous entry's memory inside one storage (and share a step count)
+    into one flat update.  Yields ``(param, grad, exp_avg, exp_avg_sq, step)``
+    as 1-D spans."""
+    runs: list[dict] = []
+    for tensors_and_step in sorted(entries, key=lambda e: e[0].data_ptr()):
+        tensors, step = tensors_and_step[:4], tensors_and_step[4]
+        if runs:
+            run = runs[-1]
+            if run["step"] == step and all(_follows(a, b) for a, b in zip(run["last"], tensors)):
+                run["numel"] += tensors[0].numel()
+                run["last"] = tensors
+                continue
+        runs.append({"first": tensors, "last": tensors, "numel": tensors[0].numel(), "step": step})
+    for run in runs:
+        yield (*(_flat_span(t, run["numel"]) for t in run["first"]), run["step"])
+
+
+def _flat_span(first: Tensor, numel: int) -> Tensor:
+    """1-D view of ``numel`` elements starting at ``first``'s first element."""
+    if first.numel() == numel:
+        return first.reshape(-1)
+    return torch.as_strided(first, (numel,), (1,), first.storage_offset())

@@ -1,0 +1,166 @@
+"""Tensor-level entry points of the HIP optimizer kernels (current stream, no synchronisation)."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import _lib
+
+NS_COEFFICIENTS = (3.4445, -4.7750, 2.0315)
+NS_EPS = 1e-7
+NS_STEPS = 5
+
+_DTYPE_CODES = {torch.float32: _lib.DT_F32, torch.bfloat16: _lib.DT_BF16}
+
+
+def adjust_lr(lr: float, adjust_lr_fn: str | None, param_shape) -> float:
+    """Muon's shape-dependent learning-rate factor (torch/optim/_muon.py:73-84)."""
+    rows, cols = param_shape[:2]
+    if adjust_lr_fn is None or adjust_lr_fn == "original":
+        ratio = math.sqrt(max(1, rows / cols))
+    elif adjust_lr_fn == "match_rms_adamw":
+        ratio = 0.2 * math.sqrt(max(rows, cols))
+    else:
+        ratio = 1.0
+    return lr * ratio
+
+
+def muon_workspace_bytes(rows: int, cols: int) -> int:
+    n = int(_lib.lib().mfsdp_muon_workspace_bytes(rows, cols))
+    if n <= 0:
+        raise ValueError("Param gradient must be a 2D matrix")
+    return n
+
+
+class MuonWorkspace:
+    """Scratch memory for the Newton-Schulz iteration, grown on demand and
+    reused across matrices (the kernels themselves never allocate)."""
+
+    def __init__(self, device) -> None:
+        self.device = torch.device(device)
+        self.buffer: torch.Tensor | None = None
+
+    def get(self, rows: int, cols: int) -> torch.Tensor:
+        need = muon_workspace_bytes(rows, cols)
+        if self.buffer is None or self.buffer.numel() < need:
+            self.buffer = None  # release before growing
+            self.buffer = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self.buffer
+
+
+def _check_matrix(t: torch.Tensor, what: str) -> None:
+    if t.ndim != 2:
+        raise ValueError("Param gradient must be a 2D matrix" if what == "grad" else f"{what} must be a 2D matrix")
+    if not t.is_cuda or not t.is_contiguous():
+        raise RuntimeError(f"{what} must be a contiguous CUDA tensor")
+    if t.dtype not in _DTYPE_CODES:
+        raise RuntimeError(f"{what} must be float32 or bfloat16, got {t.dtype}")
+
+
+def newton_schulz(
+    update: torch.Tensor,
+    ns_coefficients=NS_COEFFICIENTS,
+    ns_steps: int = NS_STEPS,
+    eps: float = NS_EPS,
+    *,
+    workspace: MuonWorkspace | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """bf16 orthogonalisation of ``update`` (torch/optim/_muon.py:31-70)."""
+    if ns_steps >= 100:
+        raise ValueError("Number of steps must be less than 100 for computational efficiency")
+    if update.ndim != 2:
+        raise ValueError("Input tensor gradient must be a 2D matrix")
+    if len(ns_coefficients) != 3:
+        raise ValueError("Coefficients must be a tuple of exactly 3 values")
+    _check_matrix(update, "update")
+    rows, cols = update.shape
+    workspace = workspace or MuonWorkspace(update.device)
+    ws = workspace.get(rows, cols)
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.bfloat16, device=update.device)
+    a, b, c = ns_coefficients
+    stream = torch.cuda.current_stream(update.device).cuda_stream
+    with torch.cuda.device(update.device):
+        _lib.check(
+            _lib.lib().mfsdp_newton_schulz(
+                update.data_ptr(), _DTYPE_CODES[update.dtype], rows, cols, a, b, c, ns_steps, eps,
+                out.data_ptr(), ws.data_ptr(), ws.numel(), stream,
+            )
+        )
+    return out
+
+
+def muon_step(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    momentum_buf: torch.Tensor,
+    *,
+    lr: float,
+    weight_decay: float,
+    momentum: float,
+    nesterov: bool,
+    ns_coefficients=NS_COEFFICIENTS,
+    ns_steps: int = NS_STEPS,
+    eps: float = NS_EPS,
+    adjust_lr_fn: str | None = None,
+    workspace: MuonWorkspace | None = None,
+) -> None:
+    """One matrix of ``_single_tensor_muon`` (torch/optim/_muon.py:285-318), in
+    place on ``param`` and ``momentum_buf``."""
+    if grad.ndim != 2:
+        raise ValueError("Param gradient must be a 2D matrix")
+    for t, what in ((param, "param"), (grad, "grad"), (momentum_buf, "momentum buffer")):
+        _check_matrix(t, what)
+    if not (param.dtype == grad.dtype == momentum_buf.dtype):
+        # Tensor.lerp_ rejects mixed dtypes; the reference's local shard, grad shard and state share one dtype
+        raise RuntimeError(f"param, grad and momentum buffer must share a dtype, got {param.dtype}, {grad.dtype}, {momentum_buf.dtype}")
+    if not (param.shape == grad.shape == momentum_buf.shape):
+        raise RuntimeError("param, grad and momentum buffer must share a shape")
+    if ns_steps >= 100:
+        raise ValueError("Number of steps must be less than 100 for computational efficiency")
+    rows, cols = param.shape
+    workspace = workspace or MuonWorkspace(param.device)
+    ws = workspace.get(rows, cols)
+    a, b, c = ns_coefficients
+    stream = torch.cuda.current_stream(param.device).cuda_stream
+    with torch.cuda.device(param.device):
+        _lib.check(
+            _lib.lib().mfsdp_muon_step(
+                param.data_ptr(), grad.data_ptr(), momentum_buf.data_ptr(), _DTYPE_CODES[param.dtype], rows, cols,
+                lr, weight_decay, momentum, int(bool(nesterov)), a, b, c, ns_steps, eps,
+                adjust_lr(lr, adjust_lr_fn, param.shape), ws.data_ptr(), ws.numel(), stream,
+            )
+        )
+
+
+def adamw_step(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    exp_avg: torch.Tensor,
+    exp_avg_sq: torch.Tensor,
+    step: int,
+    *,
+    lr: float,
+    betas=(0.9, 0.999),
+    eps: float = 1e-8,
+    weight_decay: float = 1e-2,
+) -> None:
+    """Fused AdamW over flat fp32 tensors; ``step`` is the 1-based count after
+    this update (torch/optim/adam.py:347-547)."""
+    for t, what in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+        if not t.is_cuda or not t.is_contiguous() or t.dtype != torch.float32:
+            raise RuntimeError(f"{what} must be a contiguous float32 CUDA tensor")
+        if t.numel() != param.numel():
+            raise RuntimeError(f"{what} has {t.numel()} elements, param has {param.numel()}")
+    if not grad.is_cuda or not grad.is_contiguous() or grad.dtype not in _DTYPE_CODES or grad.numel() != param.numel():
+        raise RuntimeError("grad must be a contiguous float32 or bfloat16 CUDA tensor of the param's size")
+    stream = torch.cuda.current_stream(param.device).cuda_stream
+    with torch.cuda.device(param.device):
+        _lib.check(
+            _lib.lib().mfsdp_adamw_step(
+                param.data_ptr(), grad.data_ptr(), _DTYPE_CODES[grad.dtype], exp_avg.data_ptr(), exp_avg_sq.data_ptr(),
+                param.numel(), int(step), lr, betas[0], betas[1], eps, weight_decay, stream,
+            )
+        )

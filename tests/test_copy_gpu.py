@@ -162,6 +162,17 @@ def test_copy_range_alignments():
             assert torch.count_nonzero(buf[:shift]) == 0 and torch.count_nonzero(buf[shift + n :]) == 0
 
 
+def assert_same_bf16(have: torch.Tensor, source_f32: torch.Tensor):
+    """Bit-exact with Tensor.to(bfloat16) wherever the input is a number.  NaN payloads are not
+    portable (torch's own CPU conversion gives 0xFFFF from its vector loop and 0x7FC0 from its scalar
+    tail), so NaN inputs must give the quiet NaN 0x7FC0 of the scalar conversion."""
+    expect = source_f32.to(torch.bfloat16)
+    nan = torch.isnan(source_f32)
+    got = bits(have)
+    assert torch.equal(got[~nan], bits(expect)[~nan])
+    assert torch.all(got[nan] == 0x7FC0)
+
+
 def test_cast_matches_tensor_to():
     gen = torch.Generator().manual_seed(6)
     raw = torch.randint(-(2**31), 2**31 - 1, (1 << 16,), generator=gen, dtype=torch.int64).to(torch.int32)
@@ -171,13 +182,13 @@ def test_cast_matches_tensor_to():
         for shift in (0, 1, 3):
             xs = x[shift : shift + n].contiguous()
             have = native.cast(xs.to(DEV)[:], torch.bfloat16)
-            assert_same_bits(have, xs.to(torch.bfloat16))
+            assert_same_bf16(have, xs)
             back = native.cast(have, torch.float32)
-            assert_same_bits(back, xs.to(torch.bfloat16).to(torch.float32))
+            assert_same_bits(back, have.cpu().to(torch.float32))
     # unaligned views
     base = x[:4100].to(DEV)
     view = base[1:4098]
-    assert_same_bits(native.cast(view, torch.bfloat16), x[1:4098].to(torch.bfloat16))
+    assert_same_bf16(native.cast(view, torch.bfloat16), x[1:4098])
     same = torch.ones(3, device=DEV)
     assert native.cast(same, torch.float32) is same
 
@@ -281,7 +292,7 @@ def test_hidden4096_block_layer_strided_pack_unpack():
     full = normal_flat(w.total_numel, 0.02, w.seed, torch.bfloat16)
     dev_full = full.to(DEV)
     pack = pack_program(plan, torch.bfloat16, device=DEV)
-    assert pack.num_runs == 4 * len(w.specs)  # one strided run per (parameter, rank)
+    assert pack.num_runs <= 4 * len(w.specs)  # at most one strided run per (parameter, rank)
     packed = torch.empty(4 * plan.max_shard_size, dtype=torch.bfloat16, device=DEV)
     pack.run((dev_full,), packed)
     # closed form: rank (i, j) holds the contiguous copy of each matrix's block (i, j)

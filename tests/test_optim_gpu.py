@@ -1,0 +1,149 @@
+"""Parity of the HIP Muon / AdamW kernels (through the C ABI) with the CPU oracle.
+
+Tolerances: the Muon update must be within rel-Frobenius 1e-2 of the reference arithmetic on the
+same seeded inputs (bf16 products, fp32 accumulation; only the summation order differs); AdamW is
+fp32 element-wise and must agree to 1e-6 relative."""
+import pytest
+import torch
+
+from matrix_fsdp_amd.optim import functional as F
+from oracle import optim_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MUON_TOL = 1e-2
+
+
+def rel_fro(have: torch.Tensor, want: torch.Tensor) -> float:
+    have, want = have.detach().double().cpu(), want.detach().double().cpu()
+    return float(torch.linalg.norm(have - want) / torch.linalg.norm(want))
+
+
+def max_err_over_scale(have: torch.Tensor, want: torch.Tensor) -> float:
+    """Largest element error relative to the tensor's largest magnitude (fp32 element-wise kernels
+    differ from the CPU only by fused multiply-adds: a few 1e-7 of the operand scale)."""
+    want = want.detach().double().cpu()
+    return float((have.detach().double().cpu() - want).abs().max() / want.abs().max().clamp(min=1e-300))
+
+
+def make(shape, seed, std=1e-3):
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=gen) * std
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (256, 512), (512, 256), (64, 96), (100, 36), (300, 520), (1, 7), (1024, 1024)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_newton_schulz_parity(shape, dtype):
+    u = make(shape, 11).to(dtype)
+    for steps in (0, 1, 5):
+        want = O.newton_schulz(u, steps=steps)
+        have = F.newton_schulz(u.to(DEV), ns_steps=steps)
+        assert have.dtype == torch.bfloat16 and have.shape == want.shape
+        assert rel_fro(have, want) < MUON_TOL, (shape, dtype, steps)
+
+
+def test_newton_schulz_diagonal_closed_form():
+    sigma = torch.tensor([0.9, 0.5, 0.25, 0.1, 0.01, 0.0])
+    x = torch.diag(sigma)
+    have = F.newton_schulz(x.to(DEV)).float().cpu()
+    want = O.newton_schulz(x).float()
+    assert torch.count_nonzero(have - torch.diag(torch.diag(have))) == 0
+    assert torch.allclose(torch.diag(have), torch.diag(want), atol=0.02)
+
+
+def test_newton_schulz_singular_values_land_near_one():
+    u = make((384, 640), 12)
+    sv = torch.linalg.svdvals(F.newton_schulz(u.to(DEV)).float().cpu())
+    assert sv.max() < 1.3 and sv.min() > 0.3
+
+
+def test_zero_update_stays_zero():
+    have = F.newton_schulz(torch.zeros(64, 128, device=DEV))
+    assert torch.count_nonzero(have) == 0
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (192, 192)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nesterov,adjust", [(True, None), (True, "match_rms_adamw"), (False, "original")])
+def test_muon_step_parity(shape, dtype, nesterov, adjust):
+    p0 = make(shape, 1, 0.02).to(dtype)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=nesterov, adjust_lr_fn=adjust)
+    p_cpu, buf_cpu = p0.clone(), make(shape, 2).to(dtype)
+    p_dev, buf_dev = p_cpu.to(DEV), buf_cpu.to(DEV)
+    ws = F.MuonWorkspace(DEV)
+    for step in range(2):
+        g = make(shape, 20 + step).to(dtype)
+        before = p_cpu.clone()
+        O.muon_step(p_cpu, g.clone(), buf_cpu, **kw)
+        before_dev = p_dev.clone()
+        F.muon_step(p_dev, g.to(DEV), buf_dev, workspace=ws, **kw)
+        # the parameter delta, which the orthogonalised update dominates
+        # bf16 parameters move by whole bf16 steps (2^-8 relative), so their delta and value carry that grain
+        delta_err = rel_fro(p_dev.float().cpu() - before_dev.float().cpu(), p_cpu.float() - before.float())
+        buf_ok = bool(torch.allclose(buf_dev.cpu(), buf_cpu, rtol=1e-6, atol=1e-9)) if dtype == torch.float32 else rel_fro(buf_dev.float(), buf_cpu.float()) < 4e-3
+        value_err = rel_fro(p_dev.float(), p_cpu.float())
+        assert delta_err < (MUON_TOL if dtype == torch.float32 else 0.05), delta_err
+        assert buf_ok
+        assert value_err < MUON_TOL, value_err
+        p_cpu, buf_cpu = p_dev.cpu().clone(), buf_dev.cpu().clone()  # re-sync so that steps are compared one at a time
+
+
+def test_muon_step_matches_torch_optim_muon_on_device_inputs():
+    """Same check against the optimizer class the reference instantiates (CPU execution)."""
+    shape = (512, 768)
+    p0, g, buf0 = make(shape, 1, 0.02), make(shape, 3).bfloat16().float(), make(shape, 4)
+    p_ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.Muon([p_ref], lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    opt.state[p_ref]["momentum_buffer"] = buf0.clone()
+    p_ref.grad = g.clone()
+    opt.step()
+    p, buf = p0.to(DEV), buf0.to(DEV)
+    F.muon_step(p, g.to(DEV), buf, lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    assert rel_fro(p.cpu() - p0, p_ref.detach() - p0) < MUON_TOL
+    assert torch.allclose(buf.cpu(), opt.state[p_ref]["momentum_buffer"], rtol=1e-6, atol=1e-9)
+
+
+def test_muon_argument_errors():
+    p = torch.zeros(8, 8, device=DEV)
+    with pytest.raises(ValueError, match="2D"):
+        F.muon_step(p.view(-1), p.view(-1), p.view(-1), lr=0.1, weight_decay=0.0, momentum=0.9, nesterov=True)
+    with pytest.raises(RuntimeError, match="dtype"):
+        F.muon_step(p, p.bfloat16(), p, lr=0.1, weight_decay=0.0, momentum=0.9, nesterov=True)
+    with pytest.raises(ValueError, match="less than 100"):
+        F.newton_schulz(p, ns_steps=100)
+    with pytest.raises(ValueError, match="2D"):
+        F.newton_schulz(p.view(-1))
+    with pytest.raises(RuntimeError, match="Learning rate"):
+        F.muon_step(p, p.clone(), p.clone(), lr=-1.0, weight_decay=0.0, momentum=0.9, nesterov=True)
+
+
+@pytest.mark.parametrize("n", [1, 3, 1000, 4099, 1 << 20])
+@pytest.mark.parametrize("grad_dtype", [torch.float32, torch.bfloat16])
+def test_adamw_parity(n, grad_dtype):
+    p_cpu, m_cpu, v_cpu = make((n,), 5, 0.02), torch.zeros(n), torch.zeros(n)
+    p, m, v = p_cpu.to(DEV), m_cpu.to(DEV), v_cpu.to(DEV)
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for t in (1, 2, 3):
+        g = make((n,), 30 + t).to(grad_dtype)
+        O.adamw_step(p_cpu, g.float(), m_cpu, v_cpu, t, **kw)
+        F.adamw_step(p, g.to(DEV), m, v, t, **kw)
+        assert max_err_over_scale(p, p_cpu) < 1e-6
+        assert max_err_over_scale(m, m_cpu) < 1e-6
+        assert max_err_over_scale(v, v_cpu) < 1e-6
+
+
+def test_adamw_unaligned_views_and_errors():
+    n = 1001
+    base = [torch.zeros(n + 1, device=DEV) for _ in range(3)]
+    p, m, v = (b[1:] for b in base)
+    p.copy_(make((n,), 6, 0.02))
+    g = make((n,), 7).to(DEV)
+    p_cpu, m_cpu, v_cpu = p.cpu().clone(), torch.zeros(n), torch.zeros(n)
+    O.adamw_step(p_cpu, g.cpu(), m_cpu, v_cpu, 1, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    F.adamw_step(p, g, m, v, 1, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    assert max_err_over_scale(p, p_cpu) < 1e-6
+    assert all(float(b[0]) == 0.0 for b in base)
+    with pytest.raises(RuntimeError, match="step"):
+        F.adamw_step(p, g, m, v, 0, lr=1e-3)
+    with pytest.raises(RuntimeError, match="float32"):
+        F.adamw_step(p.bfloat16(), g, m, v, 1, lr=1e-3)
