@@ -1,0 +1,333 @@
+#!/usr/bin/env python3
+"""Benchmark of the MatrixFSDP hot path on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` prints ONE JSON line.
+
+A *step* is one pass of the flat-buffer copy path over the hidden4096
+workload: for each of the 32 layer buffers (Wqkv 12288x4096, Wo 4096x4096,
+W1/W3 11008x4096, W2 4096x11008, two 4096 norm vectors; bf16; 2x2
+block-sharded for a simulated world of 4) one *pack* launch (full buffer ->
+padded all-gather buffer, every rank's strided block) and one *unpack* launch
+(gathered buffer -> full buffer).  ``value`` is the algorithmic bytes of those
+64 launches (2 B read + 2 B written per element, each way) over the wall time
+of the step, inputs resident in HBM.
+
+After the timed region the same run measures, with their own clocks and
+reported under ``legs``: the hidden2048 row-split workload (pack, unpack,
+gradient chunk-cat with bf16->fp32 cast), the owner-rank Muon update of the
+three hidden4096 matrices (ms/step and Newton-Schulz TFLOP/s by the
+reference's full-GEMM flop count) and fused AdamW.  The CPU baselines time the
+CPU oracle (a port of the reference's per-segment slice-copy loops and of
+``torch.optim.Muon``) on a bounded sample on this host's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
+NS_COEFFS = (3.4445, -4.7750, 2.0315)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=0, help="layer buffers of the hidden4096 workload (0 = all 32)")
+    ap.add_argument("--skip-legs", action="store_true", help="only the timed pack/unpack region (used under rocprofv3)")
+    ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
+    ap.add_argument("--no-launch-events", action="store_true", help="no per-launch HIP events inside the timed region")
+    return ap.parse_args()
+
+
+def median(values):
+    values = sorted(values)
+    return values[len(values) // 2]
+
+
+def event_pair(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def time_launches(torch, fn, iters, warmup):
+    """Median and mean device time of ``fn`` (HIP events on the current stream)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    pairs = [event_pair(torch) for _ in range(iters)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    times = [a.elapsed_time(b) for a, b in pairs]
+    return median(times), sum(times) / len(times)
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(
+            "bench.py measures the per-rank hot path on ONE GPU (the world of size W is simulated in memory, no "
+            f"collectives are issued); --gpus {args.gpus} is not supported.",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    import matrix_fsdp_amd  # noqa: F401
+    from matrix_fsdp_amd import _lib
+    from matrix_fsdp_amd.kernels.segment_program import grad_fill_program, pack_program, unpack_program
+    from matrix_fsdp_amd.optim import functional as F
+    from matrix_fsdp_amd.workloads import HIDDEN2048_W4, HIDDEN4096_W4_BLOCK, MUON_HIDDEN4096_SHAPES, MUON_SEED
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device.", file=sys.stderr)
+        return 2
+    _lib.lib()  # fail loudly when the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    host_threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(host_threads)
+
+    # ------------------------------------------------------------------ timed region: hidden4096 2x2 block pack + unpack
+    w = HIDDEN4096_W4_BLOCK
+    layers = args.layers or w.layers
+    plan = w.plan()
+    pack = pack_program(plan, torch.bfloat16, device=dev)
+    unpack = unpack_program(plan, torch.bfloat16, device=dev)
+    padded_numel = w.world_size * plan.max_shard_size
+    gen = torch.Generator(device=dev).manual_seed(w.seed)
+    fulls = [torch.empty(w.total_numel, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02, generator=gen) for _ in range(layers)]
+    gathered = [torch.empty(padded_numel, dtype=torch.bfloat16, device=dev) for _ in range(layers)]
+    outs = [torch.empty(w.total_numel, dtype=torch.bfloat16, device=dev) for _ in range(layers)]
+    bytes_per_launch = pack.bytes_moved
+    assert unpack.bytes_moved == bytes_per_launch == 4 * w.total_numel
+    launch_events = []
+
+    def step(record: bool) -> None:
+        for i in range(layers):
+            if record:
+                a, b = event_pair(torch)
+                a.record()
+                pack.run((fulls[i],), gathered[i])
+                b.record()
+                launch_events.append((a, b))
+            else:
+                pack.run((fulls[i],), gathered[i])
+        for i in range(layers):
+            if record:
+                a, b = event_pair(torch)
+                a.record()
+                unpack.run((gathered[i],), outs[i])
+                b.record()
+                launch_events.append((a, b))
+            else:
+                unpack.run((gathered[i],), outs[i])
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    record = not args.no_launch_events
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(record)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    step_bytes = 2 * layers * bytes_per_launch
+    value = step_bytes / (elapsed / args.steps) / 1e9
+    roundtrip_ok = all(torch.equal(o, f) for o, f in zip(outs[:2], fulls[:2]))
+    if not roundtrip_ok:
+        print("unpack(pack(x)) != x", file=sys.stderr)
+        return 1
+    if launch_events:
+        avg_launch_ms = sum(a.elapsed_time(b) for a, b in launch_events) / len(launch_events)
+    else:
+        avg_launch_ms = ms_per_step / (2 * layers)
+    achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9
+    roofline = {
+        "kernel": "segment_program_kernel<16,16> (pack / unpack of one hidden4096 layer buffer)",
+        "bound": "hbm",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "algorithmic_bytes_per_launch": bytes_per_launch,
+        "avg_launch_ms": round(avg_launch_ms, 5),
+        "launches_timed": len(launch_events),
+    }
+    result = {
+        "metric": "pack/unpack GB/s (% HBM peak); Muon NS TFLOP/s + ms/step at hidden4096",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: {layers} layer buffers x {w.total_numel} bf16 elements, 2x2 block-sharded for simulated world 4, "
+            "pack + unpack of every buffer per step (one launch per buffer each way)",
+            "bytes_per_step": step_bytes,
+            "reference_convention_GBps": round(value / 2, 1),
+        },
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "roofline": roofline,
+    }
+    del fulls, gathered, outs
+    torch.cuda.empty_cache()
+
+    legs = {}
+    if not args.skip_legs:
+        # -------------------------------------------------------------- hidden2048 row split: pack / unpack / chunk-cat + cast
+        w2 = HIDDEN2048_W4
+        plan2 = w2.plan()
+        pack2 = pack_program(plan2, torch.bfloat16, device=dev)
+        unpack2 = unpack_program(plan2, torch.bfloat16, device=dev)
+        fill2 = grad_fill_program(w2.specs, plan2.shard_sizes, plan2.rank_segments, torch.bfloat16, torch.float32, device=dev)
+        gen2 = torch.Generator(device=dev).manual_seed(w2.seed)
+        full2 = [torch.empty(w2.total_numel, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02, generator=gen2) for _ in range(w2.layers)]
+        gath2 = [torch.empty(w2.world_size * plan2.max_shard_size, dtype=torch.bfloat16, device=dev) for _ in range(w2.layers)]
+        out2 = [torch.empty(w2.total_numel, dtype=torch.bfloat16, device=dev) for _ in range(w2.layers)]
+        grads2 = [[torch.empty(s.numel, dtype=torch.bfloat16, device=dev).normal_(0.0, 1e-3, generator=gen2) for s in w2.specs] for _ in range(w2.layers)]
+        packed32 = [torch.empty(w2.world_size * plan2.max_shard_size, dtype=torch.float32, device=dev) for _ in range(w2.layers)]
+
+        def all_layers(fn):
+            def run():
+                for i in range(w2.layers):
+                    fn(i)
+            return run
+
+        for name, fn, nbytes in (
+            ("pack", all_layers(lambda i: pack2.run((full2[i],), gath2[i])), pack2.bytes_moved),
+            ("unpack", all_layers(lambda i: unpack2.run((gath2[i],), out2[i])), unpack2.bytes_moved),
+            ("chunk_cat_bf16_to_f32", all_layers(lambda i: fill2.run(grads2[i], packed32[i])), fill2.bytes_moved),
+        ):
+            med, _ = time_launches(torch, fn, 20, 5)
+            legs[f"hidden2048_w4_rows.{name}"] = {
+                "ms_all_8_layers": round(med, 4),
+                "GBps": round(w2.layers * nbytes / (med * 1e-3) / 1e9, 1),
+                "pct_hbm_peak": round(100 * w2.layers * nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+            }
+        assert torch.equal(out2[0], full2[0])
+        del full2, gath2, out2, grads2, packed32
+        torch.cuda.empty_cache()
+
+        # -------------------------------------------------------------- Muon on the hidden4096 matrices
+        ws = F.MuonWorkspace(dev)
+        genm = torch.Generator(device=dev).manual_seed(MUON_SEED)
+        mats = []
+        for shape in MUON_HIDDEN4096_SHAPES:
+            p = torch.empty(shape, device=dev).normal_(0.0, 0.02, generator=genm)
+            g = torch.empty(shape, device=dev).normal_(0.0, 1e-3, generator=genm).bfloat16().float()  # bf16-valued grads
+            buf = torch.empty(shape, device=dev).normal_(0.0, 1e-3, generator=genm)
+            mats.append((p, g, buf))
+        kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True, ns_coefficients=NS_COEFFS, ns_steps=5, eps=1e-7)
+
+        def muon_all():
+            for p, g, buf in mats:
+                F.muon_step(p, g, buf, workspace=ws, **kw)
+
+        med, _ = time_launches(torch, muon_all, 10, 3)
+        flops = 0
+        per_matrix = {}
+        for (p, g, buf), shape in zip(mats, MUON_HIDDEN4096_SHAPES):
+            m, n = min(shape), max(shape)
+            fl = 5 * (4 * m * m * n + 2 * m**3)
+            flops += fl
+            t, _ = time_launches(torch, lambda: F.muon_step(p, g, buf, workspace=ws, **kw), 10, 2)
+            per_matrix[f"{shape[0]}x{shape[1]}"] = {"ms": round(t, 4), "TFLOPs": round(fl / (t * 1e-3) / 1e12, 1)}
+        tflops = flops / (med * 1e-3) / 1e12
+        legs["muon_hidden4096"] = {
+            "ms_per_step": round(med, 4),
+            "ns_TFLOPs_reference_flop_count": round(tflops, 1),
+            "pct_bf16_mfma_peak": round(100 * tflops / BF16_MFMA_PEAK_TFLOPS, 2),
+            "flop_count": "5 * (4 m^2 n + 2 m^3) per matrix, full GEMMs as the reference executes them; the time is the whole "
+            "update (momentum, norm, Newton-Schulz, parameter update)",
+            "dtype_variant": "fp32 params / momentum, bf16-valued fp32 grads",
+            "per_matrix": per_matrix,
+        }
+        result["muon_ns_TFLOPs"] = round(tflops, 1)
+        result["muon_ms_per_step"] = round(med, 4)
+        result["roofline_muon"] = {
+            "kernel": "gemm_nt_kernel (Newton-Schulz products, whole Muon step timed)",
+            "bound": "mfma",
+            "achieved": round(tflops, 1),
+            "peak": BF16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+        }
+        del mats
+        torch.cuda.empty_cache()
+
+        # -------------------------------------------------------------- fused AdamW on a flat fp32 shard
+        n_adam = 41_062_400
+        pa, ga = torch.randn(n_adam, device=dev) * 0.02, torch.randn(n_adam, device=dev) * 1e-3
+        ma, va = torch.zeros(n_adam, device=dev), torch.zeros(n_adam, device=dev)
+        med, _ = time_launches(torch, lambda: F.adamw_step(pa, ga, ma, va, 1, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1), 20, 5)
+        legs["adamw_flat_shard_41M_fp32"] = {"ms": round(med, 4), "GBps": round(28 * n_adam / (med * 1e-3) / 1e9, 1), "pct_hbm_peak": round(100 * 28 * n_adam / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        del pa, ga, ma, va
+        result["legs"] = legs
+
+    # ------------------------------------------------------------------ CPU baselines (oracle port, bounded samples)
+    if not args.skip_cpu:
+        from oracle import copy_oracle, optim_oracle
+
+        cpu_full = torch.empty(w.total_numel, dtype=torch.bfloat16).normal_(0.0, 0.02, generator=torch.Generator().manual_seed(w.seed))
+        reps, t_cpu = 0, 0.0
+        while reps < 40 and t_cpu < 12.0:
+            t0 = time.perf_counter()
+            padded = copy_oracle.pack_to_padded(cpu_full, plan)
+            back = copy_oracle.unpack_from_padded(padded, plan)
+            t_cpu += time.perf_counter() - t0
+            reps += 1
+        assert torch.equal(back, cpu_full)
+        cpu_gbps = reps * 2 * bytes_per_launch / t_cpu / 1e9
+        result["cpu_baseline"] = {
+            "value": round(cpu_gbps, 3),
+            "unit": "GB/s",
+            "cores": host_threads,
+            "kind": "port",
+            "sample": f"{reps} x (pack + unpack) of ONE of the 32 hidden4096 layer buffers ({w.total_numel} bf16 elements, ~85k row segments) with the "
+            "oracle's per-segment slice-copy loops; same byte accounting as the GPU value",
+            "seconds": round(t_cpu, 2),
+        }
+        if not args.skip_legs:
+            u = torch.empty(4096, 4096).normal_(0.0, 1e-3, generator=torch.Generator().manual_seed(MUON_SEED))
+            fl, t_ns, ns_reps = 0, 0.0, 0
+            while ns_reps < 20 and t_ns < 10.0:
+                t0 = time.perf_counter()
+                optim_oracle.newton_schulz(u, NS_COEFFS, 5, 1e-7)
+                t_ns += time.perf_counter() - t0
+                fl += 5 * (4 * 4096**3 + 2 * 4096**3)
+                ns_reps += 1
+            result["cpu_baseline_muon"] = {
+                "value": round(fl / t_ns / 1e12, 4),
+                "unit": "TFLOP/s",
+                "cores": host_threads,
+                "kind": "port",
+                "sample": f"{ns_reps} x 5-step Newton-Schulz of one 4096x4096 matrix with the oracle (torch bf16 matmuls on the CPU)",
+                "seconds": round(t_ns, 2),
+            }
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

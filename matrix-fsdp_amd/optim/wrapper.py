@@ -1,0 +1,286 @@
+"""Optimizer construction for flat-buffer managed parameters.
+
+Mirrors the Muon / AdamW wiring of matrix_fsdp/optim/wrapper.py
+(``MixedMuonAdamWOptimizer`` :353-612, ``classify_matrix_optimizer_params``
+:687-737, ``configure_optimizer`` :763-821, ``_optimizer_type_for_param``
+:827-846) with the inner optimizers replaced by the HIP-backed ``Muon`` and
+``FusedAdamW`` of this package.  The "units" handed in are ``MatrixFlatBuffer``
+objects (or a module carrying them as ``_matrix_fsdp_flat_buffers``); the
+scheduler / lifecycle arguments of the reference have no counterpart here and
+are rejected rather than silently ignored.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Iterable
+
+import torch
+from torch import nn
+
+from ..core.managed_param import ManagedParam
+from .adamw import FusedAdamW
+from .adamw_state import initialize_flat_adamw_state
+from .muon import Muon
+
+DEFAULT_MUON_ADJUST_LR_FN = "match_rms_adamw"
+
+
+@dataclass(frozen=True)
+class MatrixOptimizerParamGroupSummary:
+    name: str
+    optimizer_type: str
+    param_fqns: tuple[str, ...]
+    numel: int
+
+    def as_dict(self) -> dict[str, Any]:
+        return {"name": self.name, "optimizer_type": self.optimizer_type, "param_fqns": self.param_fqns, "numel": self.numel}
+
+
+@dataclass(frozen=True)
+class ClassifiedMatrixOptimizerParams:
+    muon_params: tuple[nn.Parameter, ...]
+    adamw_params: tuple[nn.Parameter, ...]
+    group_summaries: tuple[MatrixOptimizerParamGroupSummary, ...]
+
+
+@dataclass(frozen=True)
+class MatrixOptimizerConfig:
+    optimizer: str = "adamw"
+    kwargs: dict[str, Any] = field(default_factory=dict)
+    default_matrix_optimizer: str = "muon"
+    default_other_optimizer: str = "adamw"
+
+
+def collect_flat_buffers(module_or_units) -> list:
+    if isinstance(module_or_units, nn.Module):
+        found = []
+        for module in module_or_units.modules():
+            found.extend(getattr(module, "_matrix_fsdp_flat_buffers", ()))
+        return found
+    if hasattr(module_or_units, "local_param_views"):
+        return [module_or_units]
+    return list(module_or_units)
+
+
+def _optimizer_type_for_param(managed_param: ManagedParam, param: nn.Parameter, *, default_matrix_optimizer: str, default_other_optimizer: str) -> str:
+    """Muon only for parameters whose *local view* is the whole 2-D matrix."""
+    hint = managed_param.shard_hint.optimizer_type
+    if hint == "muon":
+        if len(managed_param.shape) != 2 or param.ndim != 2:
+            raise ValueError(
+                f"Param {managed_param.fqn!r} is marked for Muon, but its local view is not a full 2D matrix. "
+                f"Use matrix_owner planning for Muon parameters."
+            )
+        return "muon"
+    if hint == "adamw":
+        return "adamw"
+    if len(managed_param.shape) == 2 and param.ndim == 2:
+        return default_matrix_optimizer
+    return default_other_optimizer
+
+
+def classify_matrix_optimizer_params(module_or_units, *, default_matrix_optimizer: str = "muon", default_other_optimizer: str = "adamw") -> ClassifiedMatrixOptimizerParams:
+    flat_buffers = collect_flat_buffers(module_or_units)
+    if not flat_buffers:
+        raise ValueError("Expected a module wrapped by matrix_fully_shard().")
+    if default_matrix_optimizer not in ("muon", "adamw"):
+        raise ValueError("default_matrix_optimizer must be 'muon' or 'adamw'.")
+    if default_other_optimizer not in ("muon", "adamw"):
+        raise ValueError("default_other_optimizer must be 'muon' or 'adamw'.")
+    grouped: dict[str, list[tuple[ManagedParam, nn.Parameter]]] = {"muon": [], "adamw": []}
+    seen: set[int] = set()
+    for fb in flat_buffers:
+        for view in fb.local_param_views:
+            mp = view.managed_param
+            param = mp.param
+            if id(param) in seen or param.numel() == 0:
+                continue
+            seen.add(id(param))
+            kind = _optimizer_type_for_param(mp, param, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer)
+            grouped[kind].append((mp, param))
+    if not grouped["muon"] and not grouped["adamw"]:
+        raise RuntimeError("No non-empty local MatrixFSDP parameters were found for optimizer construction.")
+    summaries = tuple(
+        MatrixOptimizerParamGroupSummary(kind, kind, tuple(mp.fqn for mp, _ in entries), sum(p.numel() for _, p in entries))
+        for kind, entries in grouped.items()
+        if entries
+    )
+    return ClassifiedMatrixOptimizerParams(
+        tuple(p for _, p in grouped["muon"]), tuple(p for _, p in grouped["adamw"]), summaries
+    )
+
+
+class MixedMuonAdamWOptimizer:
+    """Muon on local full 2-D matrices, AdamW on everything else; the two inner
+    optimizers stay separate objects.  Defaults follow the reference
+    (``muon_momentum=0.5``, ``muon_ns_steps=2``, ``muon_adjust_lr_fn="match_rms_adamw"``)."""
+
+    def __init__(
+        self,
+        muon_params: Iterable[nn.Parameter],
+        adamw_params: Iterable[nn.Parameter],
+        *,
+        group_summaries: Iterable[MatrixOptimizerParamGroupSummary] = (),
+        lr: float = 0.001,
+        weight_decay: float = 0.01,
+        muon_lr: float | None = None,
+        adamw_lr: float | None = None,
+        adamw_betas: tuple[float, float] = (0.9, 0.999),
+        adamw_eps: float = 1e-8,
+        adamw_weight_decay: float | None = None,
+        muon_weight_decay: float | None = None,
+        muon_momentum: float = 0.5,
+        muon_ns_steps: int = 2,
+        muon_adjust_lr_fn: str | None = DEFAULT_MUON_ADJUST_LR_FN,
+        flat_adamw_state: bool = False,
+        flat_buffers: Iterable | None = None,
+    ) -> None:
+        self.muon_params = tuple(p for p in muon_params if p.numel() > 0)
+        self.adamw_params = tuple(p for p in adamw_params if p.numel() > 0)
+        self.group_summaries = tuple(group_summaries)
+        self.flat_adamw_state = flat_adamw_state
+        self.flat_buffers = list(flat_buffers or ())
+        self.muon = None
+        self.adamw = None
+        if self.muon_params:
+            self.muon = Muon(
+                self.muon_params,
+                lr=lr if muon_lr is None else muon_lr,
+                momentum=muon_momentum,
+                ns_steps=muon_ns_steps,
+                weight_decay=weight_decay if muon_weight_decay is None else muon_weight_decay,
+                adjust_lr_fn=muon_adjust_lr_fn,
+            )
+        if self.adamw_params:
+            self.adamw = FusedAdamW(
+                self.adamw_params,
+                lr=lr if adamw_lr is None else adamw_lr,
+                betas=adamw_betas,
+                eps=adamw_eps,
+                weight_decay=weight_decay if adamw_weight_decay is None else adamw_weight_decay,
+            )
+        if self.muon is None and self.adamw is None:
+            raise RuntimeError("MixedMuonAdamWOptimizer requires at least one non-empty parameter.")
+
+    @property
+    def param_groups(self) -> list[dict[str, Any]]:
+        groups = []
+        for opt in (self.muon, self.adamw):
+            if opt is not None:
+                groups.extend(opt.param_groups)
+        return groups
+
+    @property
+    def state(self) -> dict[Any, Any]:
+        state = {}
+        for opt in (self.muon, self.adamw):
+            if opt is not None:
+                state.update(opt.state)
+        return state
+
+    @property
+    def defaults(self) -> dict[str, Any]:
+        return {
+            "muon": dict(self.muon.defaults) if self.muon is not None else None,
+            "adamw": dict(self.adamw.defaults) if self.adamw is not None else None,
+        }
+
+    def step(self, closure=None):
+        if closure is not None:
+            raise NotImplementedError("MixedMuonAdamWOptimizer does not support closures.")
+        if self.flat_adamw_state and self.adamw is not None and self.flat_buffers:
+            initialize_flat_adamw_state(self.adamw, self.flat_buffers)
+        result = None
+        if self.muon is not None:
+            result = self.muon.step()
+        if self.adamw is not None:
+            adamw_result = self.adamw.step()
+            result = result if result is not None else adamw_result
+        return result
+
+    def zero_grad(self, *args: Any, **kwargs: Any) -> None:
+        for opt in (self.muon, self.adamw):
+            if opt is not None:
+                opt.zero_grad(*args, **kwargs)
+
+    def state_dict(self) -> dict[str, Any]:
+        return {
+            "muon": self.muon.state_dict() if self.muon is not None else None,
+            "adamw": self.adamw.state_dict() if self.adamw is not None else None,
+            "group_summaries": tuple(g.as_dict() for g in self.group_summaries),
+        }
+
+    def load_state_dict(self, state_dict: dict[str, Any]) -> None:
+        if self.muon is not None and state_dict.get("muon") is not None:
+            self.muon.load_state_dict(state_dict["muon"])
+        if self.adamw is not None and state_dict.get("adamw") is not None:
+            self.adamw.load_state_dict(state_dict["adamw"])
+
+    def iter_named_optimizers(self) -> tuple[tuple[str, Any], ...]:
+        return tuple((name, opt) for name, opt in (("muon", self.muon), ("adamw", self.adamw)) if opt is not None)
+
+    def add_param_group(self, param_group: dict[str, Any]) -> None:
+        raise NotImplementedError("MixedMuonAdamWOptimizer does not support adding param groups after construction.")
+
+    def optimizer_group_summary(self) -> dict[str, Any]:
+        return {
+            "optimizer": "mixed_muon_adamw",
+            "has_muon": self.muon is not None,
+            "has_adamw": self.adamw is not None,
+            "groups": tuple(g.as_dict() for g in self.group_summaries),
+        }
+
+
+def make_mixed_muon_adamw_optimizer(module_or_units, *, default_matrix_optimizer: str = "muon", default_other_optimizer: str = "adamw", **optimizer_kwargs: Any) -> MixedMuonAdamWOptimizer:
+    flat_buffers = collect_flat_buffers(module_or_units)
+    classified = classify_matrix_optimizer_params(
+        flat_buffers, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer
+    )
+    return MixedMuonAdamWOptimizer(
+        classified.muon_params, classified.adamw_params, group_summaries=classified.group_summaries, flat_buffers=flat_buffers, **optimizer_kwargs
+    )
+
+
+def _local_params(module_or_units) -> list[nn.Parameter]:
+    params, seen = [], set()
+    for fb in collect_flat_buffers(module_or_units):
+        for view in fb.local_param_views:
+            p = view.managed_param.param
+            if id(p) not in seen and p.numel() > 0:
+                seen.add(id(p))
+                params.append(p)
+    return params
+
+
+def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig = "adamw", **kwargs: Any):
+    """``'adamw'`` / ``'sgd'`` / ``'muon'`` / ``'mixed_muon_adamw'`` (aliases
+    ``'muon_adamw'``, ``'mixed'``) over the local parameters of the given
+    flat buffers (matrix_fsdp/optim/wrapper.py:763-821)."""
+    default_matrix_optimizer, default_other_optimizer = "muon", "adamw"
+    optimizer_kwargs: dict[str, Any] = {}
+    if isinstance(optimizer, MatrixOptimizerConfig):
+        kind = optimizer.optimizer
+        optimizer_kwargs.update(optimizer.kwargs)
+        default_matrix_optimizer = optimizer.default_matrix_optimizer
+        default_other_optimizer = optimizer.default_other_optimizer
+    else:
+        kind = optimizer
+    optimizer_kwargs.update(kwargs)
+    default_matrix_optimizer = optimizer_kwargs.pop("default_matrix_optimizer", default_matrix_optimizer)
+    default_other_optimizer = optimizer_kwargs.pop("default_other_optimizer", default_other_optimizer)
+    kind = kind.lower()
+    if kind in ("mixed_muon_adamw", "muon_adamw", "mixed"):
+        return make_mixed_muon_adamw_optimizer(
+            module_or_units, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer, **optimizer_kwargs
+        )
+    params = _local_params(module_or_units)
+    if kind == "adamw":
+        return FusedAdamW(params, **optimizer_kwargs)
+    if kind == "sgd":
+        return torch.optim.SGD(params, **optimizer_kwargs)
+    if kind == "muon":
+        return Muon(params, **optimizer_kwargs)
+    raise ValueError(f"optimizer must be one of 'adamw', 'sgd', 'muon', or 'mixed_muon_adamw', got {kind!r}.")
+
+
+configure_matrix_optimizer = configure_optimizer
