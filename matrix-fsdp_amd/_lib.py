@@ -66,6 +66,7 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_float, c_float, c_float, c_int,
          c_float, c_float, c_float, c_int, c_float, c_float, c_void_p, c_int64, c_void_p],
     ),
+    "mfsdp_set_muon_tuning": (None, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "mfsdp_adamw_step": (
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_float, c_float, c_float, c_float, c_float, c_void_p],

@@ -31,6 +31,7 @@ struct Workspace {
   uint16_t* xraw;          // rows x cols unscaled bf16 update (aliases X[1])
   float* partials;
   float* scalars;
+  GemmScratch gemm;        // fp32 partial tiles of K-split GEMM pieces
   int64_t bytes;
 };
 
@@ -54,6 +55,8 @@ bool plan_workspace(int64_t rows, int64_t cols, void* base, Workspace* w) {
   w->B = reinterpret_cast<uint16_t*>(take(a_bytes));
   w->partials = reinterpret_cast<float*>(take(round_up(kMuonMaxPartials * 4, kAlign)));
   w->scalars = reinterpret_cast<float*>(take(kAlign));
+  w->gemm.partials = take(kGemmPartialsBytes);
+  w->gemm.partials_bytes = kGemmPartialsBytes;
   w->xraw = w->X[1];
   w->bytes = off;
   return true;
@@ -77,19 +80,19 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     g.M = w.mp; g.N = w.mp; g.K = w.np;
     g.ldp = w.np; g.ldq = w.np; g.ldd = 0; g.ldc = w.mp; g.ldct = 0;
     g.alpha = 1.0f; g.beta = 0.0f; g.symmetric = 1;
-    if (int rc = gemm_nt_bf16(g, stream)) return rc;
+    if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.A; g.Q = w.A; g.D = w.A; g.C = w.B; g.CT = nullptr;
     g.M = w.mp; g.N = w.mp; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.mp; g.ldc = w.mp; g.ldct = 0;
     g.alpha = c; g.beta = b; g.symmetric = 1;
-    if (int rc = gemm_nt_bf16(g, stream)) return rc;
+    if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.B; g.Q = w.XT[cur]; g.D = w.X[cur]; g.C = w.X[nxt]; g.CT = w.XT[nxt];
     g.M = w.mp; g.N = w.np; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.np; g.ldc = w.np; g.ldct = w.mp;
     g.alpha = 1.0f; g.beta = a; g.symmetric = 0;
-    if (int rc = gemm_nt_bf16(g, stream)) return rc;
+    if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
   }
   const int fin = steps & 1;
   *ortho = w.tall ? w.XT[fin] : w.X[fin];
@@ -152,4 +155,16 @@ extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf
   if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, &ortho, &ldo, s)) return rc;
   const float decay = static_cast<float>(1.0 - static_cast<double>(lr) * static_cast<double>(weight_decay));
   return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, decay, -adjusted_lr, s);
+}
+
+extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,
+                                      int max_splits, int stagger) {
+  GemmTuning t = get_gemm_tuning();
+  if (general_variant > 0) t.general_variant = general_variant;
+  if (symmetric_variant > 0) t.symmetric_variant = symmetric_variant;
+  if (direct_to_lds > 0) t.direct_to_lds = direct_to_lds == 1;
+  if (split_remainder > 0) t.split_remainder = split_remainder == 1;
+  if (max_splits > 0) t.max_splits = max_splits;
+  if (stagger >= 0) { t.stagger = stagger & 0xffff; t.debug = stagger >> 16; }
+  set_gemm_tuning(t);
 }

@@ -1,4 +1,4 @@
-// bf16 MFMA GEMM used by the Newton-Schulz iteration (gfx950).
+// bf16 MFMA GEMM used by the Newton-Schulz iteration (gfx950).  Internal to libmfsdp_hip.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -25,10 +25,26 @@ struct GemmNtArgs {
   int symmetric;
 };
 
-// Enqueues the GEMM on `stream`; returns an MFSDP_* status.
-int gemm_nt_bf16(const GemmNtArgs& args, hipStream_t stream);
+// Device scratch for the K-split pieces of the last partial round of tiles (fp32 partial tiles).
+struct GemmScratch {
+  void* partials = nullptr;
+  int64_t partials_bytes = 0;
+};
+constexpr int64_t kGemmPartialsBytes = 64ll << 20;
 
-// Tile variant selection for experiments: 0 = default heuristic, 1 = 256x256 tiles, 2 = 128x128 tiles.
-void set_gemm_variant(int variant);
+struct GemmTuning {
+  int general_variant = 1;    // 1: 256x256 tile / 8 waves, 2: 128x128 / 4 waves, 3: 256x256 / 4 waves
+  int symmetric_variant = 2;
+  int direct_to_lds = 1;      // stream slabs HBM -> LDS without a register round trip
+  int split_remainder = 1;    // split the tiles of the last partial round along K
+  int max_splits = 16;
+  int stagger = 0;            // K-walk start offset (slabs) between consecutive tiles; 0 = none
+  int debug = 0;              // experiments only (wrong results): bit 0 = no slab streaming after the first two
+};
+void set_gemm_tuning(const GemmTuning& tuning);
+GemmTuning get_gemm_tuning();
+
+// Enqueues the GEMM on `stream`; returns an MFSDP_* status.
+int gemm_nt_bf16(const GemmNtArgs& args, const GemmScratch& scratch, hipStream_t stream);
 
 }  // namespace mfsdp

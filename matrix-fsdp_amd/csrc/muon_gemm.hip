@@ -4,18 +4,30 @@
 // reduces to once X and X^T are both kept: X X^T, A A^T (A symmetric) and B (X^T)^T.  A workgroup owns
 // a BM x BN tile of C; its waves each own a (BM/WM) x (BN/WN) sub-tile built from 32x32x16 bf16 MFMAs
 // with fp32 accumulators.  K is walked in slabs of 64: the slab of P and Q is staged in LDS as rows of
-// 128 bytes whose eight 16-byte chunks are XOR-swizzled with the row index, so that the 128-bit
-// fragment reads of 32 consecutive rows are bank-conflict free.  Two LDS stages: the next slab is
-// fetched from HBM into registers while the current one feeds the MFMAs.
+// 128 bytes whose eight 16-byte chunks are XOR-swizzled with (row / 2) % 8: the LDS has 64 banks of 4
+// bytes, two rows span them once, so any 16 consecutive rows read at one logical chunk touch every bank
+// exactly once and the 128-bit fragment reads are bank-conflict free.  Two LDS stages: the next slab streams
+// from HBM straight into LDS (global_load ... lds, no register round trip) while the current one feeds
+// the MFMAs.
+//
+// Tile scheduling.  Tiles are handed to workgroups so that the groups sharing an XCD (block ids
+// congruent mod 8) work on neighbouring tiles and reuse that XCD's L2.  When the tile count is not a
+// multiple of the number of resident workgroups, the tiles of the last, partial round are split along
+// K into pieces that fill the machine once more for a fraction of a tile's time; each piece leaves an
+// fp32 partial tile in a workspace and a small fix-up kernel sums the pieces in split order and runs
+// the epilogue (the kernel boundary is the only synchronisation: no fences, no spinning).
 #include "muon_gemm.h"
 
 #include "mfsdp_common.h"
+
+#include <algorithm>
 
 namespace mfsdp {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -31,16 +43,20 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
-// Maps the hardware block id to a tile so that (a) the blocks that land on one XCD (ids congruent
-// mod 8) work on a contiguous range of logical tiles and share that XCD's L2, and (b) consecutive
-// logical tiles walk down GROUP_M tile rows before moving to the next tile column.
+struct Schedule {
+  int tiles_m, tiles_n;
+  int full_tiles;   // tiles computed whole, one per workgroup (block ids [0, full_tiles))
+  int splits;       // K pieces per remaining tile (block ids from full_tiles on); 1 when nothing remains
+  float* partials;  // [remaining tiles][splits][BM][BN] fp32
+  int stagger;      // tile t starts its K walk (t * stagger) slabs in and wraps around; 0 = every tile starts at slab 0
+  int debug;        // experiments only: bit 0 = skip the HBM -> LDS streaming after the first two slabs
+};
+
+// logical tile index -> (tm, tn)
 template <int GROUP_M>
-__device__ __forceinline__ void tile_of_block(int block, int n_blocks, int tiles_m, int tiles_n, bool symmetric,
-                                              int* tm, int* tn) {
-  int logical = block;
-  if (n_blocks % kXcds == 0) logical = (block % kXcds) * (n_blocks / kXcds) + block / kXcds;
+__device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_n, bool symmetric, int* tm, int* tn) {
   if (symmetric) {
-    // logical enumerates the lower triangle row by row: t = i(i+1)/2 + j, j <= i
+    // the lower triangle row by row: t = i(i+1)/2 + j, j <= i
     int i = static_cast<int>((__fsqrt_rn(8.0f * static_cast<float>(logical) + 1.0f) - 1.0f) * 0.5f);
     while ((i + 1) * (i + 2) / 2 <= logical) ++i;
     while (i * (i + 1) / 2 > logical) --i;
@@ -48,6 +64,7 @@ __device__ __forceinline__ void tile_of_block(int block, int n_blocks, int tiles
     *tn = logical - i * (i + 1) / 2;
     return;
   }
+  // GROUP_M tile rows at a time, walking down the rows before moving to the next tile column
   const int per_group = GROUP_M * tiles_n;
   const int group = logical / per_group;
   const int first_m = group * GROUP_M;
@@ -57,10 +74,11 @@ __device__ __forceinline__ void tile_of_block(int block, int n_blocks, int tiles
   *tn = in_group / rows;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool DIRECT>
 __global__ void __launch_bounds__(WM * WN * 64)
-gemm_nt_kernel(GemmNtArgs a, int tiles_m, int tiles_n) {
+gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kThreads = WM * WN * 64;
+  constexpr int kWaves = WM * WN;
   constexpr int kWaveM = BM / WM;     // rows of C per wave
   constexpr int kWaveN = BN / WN;
   constexpr int TM = kWaveM / 32;     // 32x32 MFMA tiles per wave
@@ -73,10 +91,37 @@ gemm_nt_kernel(GemmNtArgs a, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
 
+  // ---- which tile, which K range
+  const int block = blockIdx.x;
+  const bool whole = block < sched.full_tiles;
+  int logical, split = 0, piece_tile = 0;
+  if (whole) {
+    logical = block;
+    if (sched.full_tiles % kXcds == 0) logical = (block % kXcds) * (sched.full_tiles / kXcds) + block / kXcds;
+  } else {
+    const int piece = block - sched.full_tiles;
+    piece_tile = piece / sched.splits;
+    split = piece - piece_tile * sched.splits;
+    logical = sched.full_tiles + piece_tile;
+  }
   int tm, tn;
-  tile_of_block<4>(blockIdx.x, gridDim.x, tiles_m, tiles_n, a.symmetric != 0, &tm, &tn);
+  tile_coords<4>(logical, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
   const int row0 = tm * BM;
   const int col0 = tn * BN;
+  const int k_slabs_total = a.K / kBK;
+  const int ks_begin = whole ? 0 : static_cast<int>(static_cast<int64_t>(k_slabs_total) * split / sched.splits);
+  const int ks_end = whole ? k_slabs_total : static_cast<int>(static_cast<int64_t>(k_slabs_total) * (split + 1) / sched.splits);
+
+  // Tiles that run at the same time walk K from different starting slabs: with power-of-two leading
+  // dimensions every row of a slab maps to the same memory channel, and tiles marching in lock step would all
+  // queue on that one channel.
+  const int n_slabs = ks_end - ks_begin;
+  const int k_start = (sched.stagger > 0 && n_slabs > 0) ? static_cast<int>((static_cast<int64_t>(logical) * sched.stagger) % n_slabs) : 0;
+  auto k0_of = [&](int i) {
+    int slab = i + k_start;
+    if (slab >= n_slabs) slab -= n_slabs;
+    return (ks_begin + slab) * kBK;
+  };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -87,34 +132,62 @@ gemm_nt_kernel(GemmNtArgs a, int tiles_m, int tiles_n) {
   const __bf16* __restrict__ P = static_cast<const __bf16*>(a.P) + static_cast<int64_t>(row0) * a.ldp;
   const __bf16* __restrict__ Q = static_cast<const __bf16*>(a.Q) + static_cast<int64_t>(col0) * a.ldq;
 
-  // slab chunk c = i * kThreads + tid  ->  row c / 8, 16-byte chunk c % 8
-  u32x4 pre_p[kPChunks], pre_q[kQChunks];
+  // ---- slab loaders.  Chunk c of a slab = row c / 8, 16-byte chunk c % 8, stored at chunk (c%8) ^ ((row/2)%8).
+  // Register-staged: thread t handles chunks i*kThreads + t.
+  u32x4 pre_p[DIRECT ? 1 : kPChunks], pre_q[DIRECT ? 1 : kQChunks];
   auto fetch = [&](int k0) {
+    if constexpr (!DIRECT) {
 #pragma unroll
-    for (int i = 0; i < kPChunks; ++i) {
-      const int c = i * kThreads + tid;
-      pre_p[i] = *reinterpret_cast<const u32x4*>(P + static_cast<int64_t>(c >> 3) * a.ldp + k0 + (c & 7) * 8);
-    }
+      for (int i = 0; i < kPChunks; ++i) {
+        const int c = i * kThreads + tid;
+        pre_p[i] = *reinterpret_cast<const u32x4*>(P + static_cast<int64_t>(c >> 3) * a.ldp + k0 + (c & 7) * 8);
+      }
 #pragma unroll
-    for (int i = 0; i < kQChunks; ++i) {
-      const int c = i * kThreads + tid;
-      pre_q[i] = *reinterpret_cast<const u32x4*>(Q + static_cast<int64_t>(c >> 3) * a.ldq + k0 + (c & 7) * 8);
+      for (int i = 0; i < kQChunks; ++i) {
+        const int c = i * kThreads + tid;
+        pre_q[i] = *reinterpret_cast<const u32x4*>(Q + static_cast<int64_t>(c >> 3) * a.ldq + k0 + (c & 7) * 8);
+      }
     }
   };
   auto stash = [&](int stage) {
-    __bf16* sp = smem + stage * kStageElems;
-    __bf16* sq = sp + BM * kBK;
+    if constexpr (!DIRECT) {
+      __bf16* sp = smem + stage * kStageElems;
+      __bf16* sq = sp + BM * kBK;
 #pragma unroll
-    for (int i = 0; i < kPChunks; ++i) {
-      const int c = i * kThreads + tid;
-      const int r = c >> 3;
-      *reinterpret_cast<u32x4*>(sp + r * kBK + (((c & 7) ^ (r & 7)) << 3)) = pre_p[i];
+      for (int i = 0; i < kPChunks; ++i) {
+        const int c = i * kThreads + tid;
+        const int r = c >> 3;
+        *reinterpret_cast<u32x4*>(sp + r * kBK + (((c & 7) ^ ((r >> 1) & 7)) << 3)) = pre_p[i];
+      }
+#pragma unroll
+      for (int i = 0; i < kQChunks; ++i) {
+        const int c = i * kThreads + tid;
+        const int r = c >> 3;
+        *reinterpret_cast<u32x4*>(sq + r * kBK + (((c & 7) ^ ((r >> 1) & 7)) << 3)) = pre_q[i];
+      }
     }
+  };
+  // Direct to LDS: one wave-level load fills 1 KiB = 8 rows; lane l lands at row l/8, chunk position l%8 and
+  // therefore fetches the global chunk that the swizzle maps there.  Wave w takes the 8-row groups w, w + kWaves, ...
+  const int dl_row = lane >> 3;
+  auto stream_in = [&](int k0, int stage) {
+    if constexpr (DIRECT) {
+      __bf16* sp = smem + stage * kStageElems;
+      __bf16* sq = sp + BM * kBK;
 #pragma unroll
-    for (int i = 0; i < kQChunks; ++i) {
-      const int c = i * kThreads + tid;
-      const int r = c >> 3;
-      *reinterpret_cast<u32x4*>(sq + r * kBK + (((c & 7) ^ (r & 7)) << 3)) = pre_q[i];
+      for (int i = 0; i < BM / 8 / kWaves; ++i) {
+        const int r0 = (i * kWaves + wave) * 8;
+        const int dl_chunk = (lane & 7) ^ (((r0 + dl_row) >> 1) & 7);
+        const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + dl_chunk * 8;
+        __builtin_amdgcn_global_load_lds(src, sp + r0 * kBK, 16, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < BN / 8 / kWaves; ++i) {
+        const int r0 = (i * kWaves + wave) * 8;
+        const int dl_chunk = (lane & 7) ^ (((r0 + dl_row) >> 1) & 7);
+        const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + dl_chunk * 8;
+        __builtin_amdgcn_global_load_lds(src, sq + r0 * kBK, 16, 0, 0);
+      }
     }
   };
 
@@ -129,102 +202,280 @@ gemm_nt_kernel(GemmNtArgs a, int tiles_m, int tiles_n) {
   const int frag_row = lane & 31;   // row of the 32-row MFMA operand this lane supplies
   const int frag_half = lane >> 5;  // which 8 of the 16 k values
 
-  const int k_slabs = a.K / kBK;
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (int ks = 0; ks < k_slabs; ++ks) {
-    const int stage = ks & 1;
-    if (ks + 1 < k_slabs) fetch((ks + 1) * kBK);
-    const __bf16* sp = smem + stage * kStageElems + (wave_m * kWaveM) * kBK;
-    const __bf16* sq = smem + stage * kStageElems + BM * kBK + (wave_n * kWaveN) * kBK;
+  // LDS offsets of this lane's fragment chunk for the four k16 steps of a slab (the row part of the
+  // swizzle only depends on frag_row, every 32-row block starts at a multiple of 16 rows)
+  const __bf16* frag_p = smem + (wave_m * kWaveM + frag_row) * kBK;
+  const __bf16* frag_q = smem + BM * kBK + (wave_n * kWaveN + frag_row) * kBK;
+  auto load_frags = [&](int stage, int kk, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
+    const int off = stage * kStageElems + (((kk * 2 + frag_half) ^ ((frag_row >> 1) & 7)) << 3);
 #pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      const int chunk = kk * 2 + frag_half;
-      bf16x8 fa[TM], fb[TN];
+    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 32 * kBK);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int r = i * 32 + frag_row;
-        fa[i] = *reinterpret_cast<const bf16x8*>(sp + r * kBK + ((chunk ^ (r & 7)) << 3));
-      }
+    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 32 * kBK);
+  };
+  auto multiply = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int r = j * 32 + frag_row;
-        fb[j] = *reinterpret_cast<const bf16x8*>(sq + r * kBK + ((chunk ^ (r & 7)) << 3));
-      }
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  };
+
+  if constexpr (DIRECT) {
+    // Software pipeline.  Fragments are double buffered in registers: the six (TM + TN) 128-bit LDS reads of
+    // step kk+1 are issued before the MFMAs of step kk, so their latency hides behind TM*TN MFMAs.  The one
+    // barrier per slab sits before the slab's last k16 step: by then every wave has its last fragments of the
+    // current stage in registers (the stage can be refilled) and its share of the next stage has landed, so
+    // the first fragments of the next slab are fetched under the last MFMAs of this one.
+    bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    if (n_slabs > 0) {
+      stream_in(k0_of(0), 0);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's chunks of the first slab are in LDS
+      __syncthreads();
+      if (n_slabs > 1) stream_in(k0_of(1), 1);
+      load_frags(0, 0, fa0, fb0);
     }
-    if (ks + 1 < k_slabs) stash(stage ^ 1);
-    __syncthreads();
+    // The fragments a k16 step multiplies were requested one step earlier; waiting for them BEFORE the next
+    // step's reads are issued costs nothing and leaves those reads a whole step of MFMAs to complete.
+    constexpr int kWaitLds = 0xC07F;  // s_waitcnt lgkmcnt(0), vmcnt / expcnt fields at their maxima
+    for (int it = 0; it < n_slabs; ++it) {
+      const int stage = it & 1;
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      load_frags(stage, 1, fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      load_frags(stage, 2, fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      load_frags(stage, 3, fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): last fragments in registers, next stage landed
+      if (it + 1 < n_slabs) {
+        __syncthreads();
+        if (it + 2 < n_slabs && !(sched.debug & 1)) stream_in(k0_of(it + 2), stage);
+        load_frags(stage ^ 1, 0, fa0, fb0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    if (n_slabs > 0) {
+      fetch(k0_of(0));
+      stash(0);
+      __syncthreads();
+    }
+    for (int it = 0; it < n_slabs; ++it) {
+      const int stage = it & 1;
+      if (it + 1 < n_slabs) fetch(k0_of(it + 1));
+#pragma unroll
+      for (int kk = 0; kk < kBK / 16; ++kk) {
+        bf16x8 fa[TM], fb[TN];
+        load_frags(stage, kk, fa, fb);
+        multiply(fa, fb);
+      }
+      if (it + 1 < n_slabs) stash(stage ^ 1);
+      __syncthreads();
+    }
   }
 
-  // Epilogue.  Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
+  // ---- K pieces: park the fp32 partial tile (row-major BM x BN); the fix-up kernel sums the pieces and
+  // runs the epilogue.  Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
+  if (!whole) {
+    float* mine = sched.partials + (static_cast<int64_t>(piece_tile) * sched.splits + split) * (BM * BN);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = wave_n * kWaveN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wave_m * kWaveM + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+          __builtin_nontemporal_store(acc[i][j][r], mine + row * BN + col);
+        }
+      }
+    return;
+  }
+
+  if (sched.debug & 2) return;  // experiments only: no epilogue
+
+  // ---- epilogue, staged through LDS so that HBM only sees whole 16-byte-per-lane, row-contiguous accesses.
+  // Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile: written
+  // straight from registers that would be 2-byte stores for C and 8-byte stores scattered over 32 rows for
+  // the transpose.  Instead: D tile -> LDS (coalesced), combine, C tile -> LDS -> HBM, transposed tile -> LDS -> HBM.
   const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
   uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
   int ldct = a.ldct;
-  if (a.symmetric && tm != tn) {  // mirror the off-diagonal tile
-    CT = C;
+  if (a.symmetric) {  // mirror the off-diagonal tile
+    CT = tm != tn ? C : nullptr;
     ldct = a.ldc;
-  } else if (a.symmetric) {
-    CT = nullptr;
   }
+  uint16_t* stage_c = reinterpret_cast<uint16_t*>(smem_raw);
+  constexpr int kLdS = BN + 8;  // row pitch of the staged C tile (elements); +8 keeps rows 16-byte aligned and skews banks
+  constexpr int kLdT = BM + 8;  // row pitch of the staged transposed tile
+  constexpr int kRowChunks = BN / 8, kColChunks = BM / 8;
+  __syncthreads();  // every wave is done reading the slab stages
+  if (D != nullptr) {
+    for (int c = tid; c < BM * kRowChunks; c += kThreads) {
+      const int r = c / kRowChunks, cc = c - r * kRowChunks;
+      *reinterpret_cast<u32x4*>(stage_c + r * kLdS + cc * 8) =
+          *reinterpret_cast<const u32x4*>(D + static_cast<int64_t>(row0 + r) * a.ldd + col0 + cc * 8);
+    }
+    __syncthreads();
+  }
+  const int lcol = wave_n * kWaveN + (lane & 31);
+  const int lrow = wave_m * kWaveM + frag_half * 4;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = col0 + wave_n * kWaveN + j * 32 + (lane & 31);
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float v = a.alpha * acc[i][j][r];
+        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32]);
+        acc[i][j][r] = v;
+      }
+  if (D != nullptr) __syncthreads();  // the D tile has been consumed
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32] =
+            __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
+  __syncthreads();
+  for (int c = tid; c < BM * kRowChunks; c += kThreads) {
+    const int r = c / kRowChunks, cc = c - r * kRowChunks;
+    *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(row0 + r) * a.ldc + col0 + cc * 8) =
+        *reinterpret_cast<const u32x4*>(stage_c + r * kLdS + cc * 8);
+  }
+  if (CT == nullptr) return;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int row = row0 + wave_m * kWaveM + i * 32 + q * 8 + frag_half * 4;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = a.alpha * acc[i][j][q * 4 + e];
-          if (D != nullptr) v[e] += a.beta * bf16_bits_to_float(D[static_cast<int64_t>(row + e) * a.ldd + col]);
-        }
-        const uint32_t lo = pack_bf16x2(v[0], v[1]);
-        const uint32_t hi = pack_bf16x2(v[2], v[3]);
-        C[static_cast<int64_t>(row) * a.ldc + col] = static_cast<uint16_t>(lo);
-        C[static_cast<int64_t>(row + 1) * a.ldc + col] = static_cast<uint16_t>(lo >> 16);
-        C[static_cast<int64_t>(row + 2) * a.ldc + col] = static_cast<uint16_t>(hi);
-        C[static_cast<int64_t>(row + 3) * a.ldc + col] = static_cast<uint16_t>(hi >> 16);
-        if (CT != nullptr) {
-          u32x2 packed = {lo, hi};
-          *reinterpret_cast<u32x2*>(CT + static_cast<int64_t>(col) * ldct + row) = packed;
-        }
+        u32x2 four = {pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]), pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3])};
+        *reinterpret_cast<u32x2*>(stage_c + (lcol + j * 32) * kLdT + lrow + i * 32 + q * 8) = four;
       }
-    }
+  __syncthreads();
+  for (int c = tid; c < BN * kColChunks; c += kThreads) {
+    const int r = c / kColChunks, cc = c - r * kColChunks;
+    *reinterpret_cast<u32x4*>(CT + static_cast<int64_t>(col0 + r) * ldct + row0 + cc * 8) =
+        *reinterpret_cast<const u32x4*>(stage_c + r * kLdT + cc * 8);
   }
 }
 
-int g_variant = 0;
+// Sums the K pieces of every split tile in split order and applies the epilogue of gemm_nt_kernel.
+template <int BM, int BN>
+__global__ void __launch_bounds__(256)
+splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
+  constexpr int kGroupsPerTile = BM * BN / 4;  // float4 groups along a row
+  const int tile = blockIdx.x / (kGroupsPerTile / 256);
+  const int group = (blockIdx.x % (kGroupsPerTile / 256)) * 256 + threadIdx.x;
+  const int lrow = group / (BN / 4);
+  const int lcol = (group % (BN / 4)) * 4;
+  int tm, tn;
+  tile_coords<4>(sched.full_tiles + tile, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
+  const int row = tm * BM + lrow;
+  const int col = tn * BN + lcol;
+  const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
+  f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int s = 0; s < sched.splits; ++s)
+    sum += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN)));
+  const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
+  uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
+  uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
+  int ldct = a.ldct;
+  if (a.symmetric) {
+    CT = tm != tn ? C : nullptr;
+    ldct = a.ldc;
+  }
+  float v[4] = {a.alpha * sum.x, a.alpha * sum.y, a.alpha * sum.z, a.alpha * sum.w};
+  if (D != nullptr) {
+    const u32x2 d = *reinterpret_cast<const u32x2*>(D + static_cast<int64_t>(row) * a.ldd + col);
+    v[0] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x));
+    v[1] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x >> 16));
+    v[2] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y));
+    v[3] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y >> 16));
+  }
+  const uint32_t lo = pack_bf16x2(v[0], v[1]);
+  const uint32_t hi = pack_bf16x2(v[2], v[3]);
+  u32x2 packed = {lo, hi};
+  *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
+  if (CT != nullptr) {
+    CT[static_cast<int64_t>(col) * ldct + row] = static_cast<uint16_t>(lo);
+    CT[static_cast<int64_t>(col + 1) * ldct + row] = static_cast<uint16_t>(lo >> 16);
+    CT[static_cast<int64_t>(col + 2) * ldct + row] = static_cast<uint16_t>(hi);
+    CT[static_cast<int64_t>(col + 3) * ldct + row] = static_cast<uint16_t>(hi >> 16);
+  }
+}
 
-template <int BM, int BN, int WM, int WN>
-int launch(const GemmNtArgs& a, hipStream_t stream) {
-  const int tiles_m = a.M / BM, tiles_n = a.N / BN;
-  const int blocks = a.symmetric ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
-  constexpr size_t smem = 2 * static_cast<size_t>(BM + BN) * kBK * sizeof(uint16_t);
-  auto kernel = gemm_nt_kernel<BM, BN, WM, WN>;
+GemmTuning g_tuning;
+
+template <int BM, int BN, int WM, int WN, bool DIRECT>
+int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, hipStream_t stream) {
+  Schedule s{};
+  s.tiles_m = a.M / BM;
+  s.tiles_n = a.N / BN;
+  const int tiles = a.symmetric ? s.tiles_m * (s.tiles_m + 1) / 2 : s.tiles_m * s.tiles_n;
+  const int slots = device_cu_count() * blocks_per_cu;
+  const int k_slabs = a.K / kBK;
+  s.full_tiles = tiles;
+  s.splits = 1;
+  s.partials = static_cast<float*>(scratch.partials);
+  s.stagger = g_tuning.stagger;
+  s.debug = g_tuning.debug;
+  const int rem = tiles % slots;
+  if (g_tuning.split_remainder && rem != 0 && scratch.partials != nullptr) {
+    // fill the machine once more with pieces of the leftover tiles; cap the pieces per tile so that the summing stays short
+    int splits = std::min({slots / rem, k_slabs, g_tuning.max_splits});
+    const int64_t tile_bytes = static_cast<int64_t>(BM) * BN * 4;
+    while (splits > 1 && static_cast<int64_t>(rem) * splits * tile_bytes > scratch.partials_bytes) --splits;
+    if (splits > 1) {
+      s.full_tiles = tiles - rem;
+      s.splits = splits;
+    }
+  }
+  const int blocks = s.full_tiles + (tiles - s.full_tiles) * s.splits;
+  constexpr size_t smem_loop = 2 * static_cast<size_t>(BM + BN) * kBK * sizeof(uint16_t);
+  constexpr size_t smem_epilogue = static_cast<size_t>(BM > BN ? BM : BN) * ((BM > BN ? BM : BN) + 8) * sizeof(uint16_t);
+  constexpr size_t smem = smem_loop > smem_epilogue ? smem_loop : smem_epilogue;
+  auto kernel = gemm_nt_kernel<BM, BN, WM, WN, DIRECT>;
   static bool configured = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!configured) {
     MFSDP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(smem)));
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WM * WN * 64), smem, stream, a, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WM * WN * 64), smem, stream, a, s);
   MFSDP_CHECK_LAUNCH("gemm_nt_kernel");
+  if (s.splits > 1) {
+    const int fix_blocks = (tiles - s.full_tiles) * (BM * BN / 4 / 256);
+    hipLaunchKernelGGL((splitk_fixup_kernel<BM, BN>), dim3(fix_blocks), dim3(256), 0, stream, a, s);
+    MFSDP_CHECK_LAUNCH("splitk_fixup_kernel");
+  }
   return MFSDP_OK;
 }
 
 }  // namespace
 
-void set_gemm_variant(int variant) { g_variant = variant; }
+void set_gemm_tuning(const GemmTuning& t) { g_tuning = t; }
+GemmTuning get_gemm_tuning() { return g_tuning; }
 
-int gemm_nt_bf16(const GemmNtArgs& a, hipStream_t stream) {
+int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kBK)
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kBK);
   if (a.symmetric && a.M != a.N) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric product needs M == N");
@@ -233,14 +484,19 @@ int gemm_nt_bf16(const GemmNtArgs& a, hipStream_t stream) {
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: leading dimension smaller than the row length");
   if ((a.ldp | a.ldq) % 8 || (reinterpret_cast<uintptr_t>(a.P) | reinterpret_cast<uintptr_t>(a.Q)) % 16)
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: operands must be 16-byte aligned with leading dimensions multiple of 8");
-  if (a.CT && ((a.ldct % 4) || reinterpret_cast<uintptr_t>(a.CT) % 8))
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: transposed output must be 8-byte aligned");
-  if (a.symmetric && ((a.ldc % 4) || reinterpret_cast<uintptr_t>(a.C) % 8))
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric output must be 8-byte aligned");
-  int variant = g_variant;
-  if (variant == 0) variant = a.symmetric ? 2 : 1;
-  if (variant == 2) return launch<128, 128, 2, 2>(a, stream);
-  return launch<256, 256, 2, 4>(a, stream);
+  if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
+      (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
+  const int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
+  const bool direct = g_tuning.direct_to_lds != 0;
+  switch (variant) {
+    case 2:  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
+      return direct ? launch<128, 128, 2, 2, true>(a, scratch, 2, stream) : launch<128, 128, 2, 2, false>(a, scratch, 2, stream);
+    case 3:  // 256x256 tile, 4 waves of 128x128
+      return direct ? launch<256, 256, 2, 2, true>(a, scratch, 1, stream) : launch<256, 256, 2, 2, false>(a, scratch, 1, stream);
+    default:  // 256x256 tile, 8 waves of 128x64
+      return direct ? launch<256, 256, 2, 4, true>(a, scratch, 1, stream) : launch<256, 256, 2, 4, false>(a, scratch, 1, stream);
+  }
 }
 
 }  // namespace mfsdp

@@ -1,0 +1,203 @@
+"""CPU tests of the host-side mirror: shard metadata, layout classification, closed-form plans, the
+C-ABI library's symbols, and the run compiler (host part of the library)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from matrix_fsdp_amd import LayoutSegment, ShardPlan, _lib, managed_params_from_named, validate_shard_plan
+from matrix_fsdp_amd.core.plans import (
+    block_grid_plan,
+    contiguous_even_plan,
+    fsdp2_chunk_plan,
+    rank_major_owner_order,
+    whole_param_owner_plan,
+)
+from matrix_fsdp_amd.kernels.segment_fusion import coalesce_contiguous_segments, coalesce_rank_segments
+from matrix_fsdp_amd.kernels.segment_program import fill_runs_for_gaps, grad_fill_runs, make_runs, merge_runs
+from matrix_fsdp_amd.runtime.grad_bucket import BucketParamGrad, MatrixGradBucket, classify_copy_in_layout, fill_reduce_scatter_input
+from matrix_fsdp_amd.runtime.param_buffer_layout import ParamBufferLayout, rank_chunk_shard_sizes
+from matrix_fsdp_amd.workloads import HIDDEN2048_W4, HIDDEN4096_W4_BLOCK, MLP_W2, param_specs
+from oracle import copy_oracle as O
+from tests.conftest import segs
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def managed(pairs):
+    return managed_params_from_named([(n, torch.nn.Parameter(torch.zeros(k))) for n, k in pairs])
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "mfsdp_hip.h")).read()
+    declared = set(re.findall(r"\b(mfsdp_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    handle = _lib.lib()
+    for name in declared:
+        assert getattr(handle, name) is not None
+    assert handle.mfsdp_abi_version() == _lib.ABI_VERSION
+    assert ctypes.sizeof(_lib.CopyRun) == 56
+
+
+def test_layout_segment_and_plan_defaults():
+    seg = LayoutSegment(3, 8, 2)
+    assert seg.numel == 5 and seg.local_end == 7 and seg.intersects(7, 9) and not seg.intersects(8, 9)
+    plan = ShardPlan(10, (4, 6), (0, 4))
+    assert plan.rank_segments == ((LayoutSegment(0, 4, 0),), (LayoutSegment(4, 10, 0),))
+    assert plan.local_range(1) == (4, 10) and plan.rank_packed_offset(1) == 4
+    validate_shard_plan(plan)
+    with pytest.raises(ValueError):
+        validate_shard_plan(ShardPlan(10, (4, 5), (0, 4)))
+    with pytest.raises(ValueError):
+        validate_shard_plan(ShardPlan.from_rank_segments(6, ((LayoutSegment(0, 4, 0),), (LayoutSegment(3, 6, 0),))))
+    with pytest.raises(ValueError):
+        validate_shard_plan(ShardPlan(4, (4,), (0,), ((LayoutSegment(0, 4, 1),),)))
+
+
+def test_managed_params_offsets_and_duplicates():
+    mps = managed([("w", 6), ("b", 4)])
+    assert [(m.fqn, m.offset, m.end, m.numel) for m in mps] == [("w", 0, 6, 6), ("b", 6, 10, 4)]
+    assert mps[0].shard_hint.optimizer_type is None and mps[1].local_name == "b"
+    with pytest.raises(ValueError, match="Duplicate"):
+        managed([("w", 1), ("w", 2)])
+    lin = torch.nn.Linear(3, 2)
+    tied = torch.nn.ModuleList([lin, lin])
+    from matrix_fsdp_amd import managed_params_from_module
+
+    assert [m.fqn for m in managed_params_from_module(lin)] == ["weight", "bias"]
+    with pytest.raises(NotImplementedError, match="shared"):
+        managed_params_from_module(tied)
+
+
+def test_coalesce_reference_vector(golden):
+    g = golden["coalesce_contiguous_segments"]
+    have = coalesce_contiguous_segments(tuple(LayoutSegment(*t) for t in g["segments"]))
+    assert have == tuple(LayoutSegment(*t) for t in g["fused"])
+    assert coalesce_contiguous_segments(()) == ()
+    assert coalesce_rank_segments(((LayoutSegment(0, 1, 0), LayoutSegment(1, 2, 1)), ())) == ((LayoutSegment(0, 2, 0),), ())
+
+
+def test_rank_chunk_detection_reference_vectors(golden):
+    for case in golden["rank_chunk_shard_sizes"]["cases"]:
+        want = None if case["shard_sizes"] is None else tuple(case["shard_sizes"])
+        assert rank_chunk_shard_sizes(segs(case["rank_segments"])) == want
+
+
+def test_param_buffer_layout_reference_vectors(golden):
+    g = golden["param_buffer_layout"]
+    layout = ParamBufferLayout(g["total_numel"], tuple(g["shard_sizes"]), segs(g["rank_segments"]))
+    assert layout.padded_numel == g["padded_numel"] and layout.padding_waste_numel == g["padding_waste_numel"]
+    assert layout.padding_waste_ratio == pytest.approx(g["padding_waste_ratio"])
+    assert layout.owner_imbalance_ratio == pytest.approx(g["owner_imbalance_ratio"])
+    assert layout.segment_count == g["segment_count"] and layout.max_segments_per_rank == g["max_segments_per_rank"]
+    assert layout.rank_chunk_fast_path and layout.packed_rank_shards_are_full_tensor_order
+    assert layout.rank_chunk_workspace_numel(compact=True) == 10 and layout.rank_chunk_workspace_numel(compact=False) == 12
+    g = golden["param_buffer_layout_not_chunks"]
+    layout = ParamBufferLayout(g["total_numel"], tuple(g["shard_sizes"]), segs(g["rank_segments"]))
+    assert not layout.rank_chunk_fast_path and not layout.packed_rank_shards_are_full_tensor_order
+
+
+@pytest.mark.parametrize("case", ["grad_bucket_padded_rank_major", "grad_bucket_flat_cat", "grad_bucket_chunk_cat"])
+def test_classify_copy_in_layout_reference_vectors(golden, case):
+    g = golden[case]
+    mps = managed(g["params"])
+    bucket = MatrixGradBucket(
+        tuple(BucketParamGrad(m, torch.tensor(v, dtype=torch.float32)) for m, v in zip(mps, g["grads"])),
+        g["total_numel"], tuple(g["shard_sizes"]), segs(g["rank_segments"]),
+    )
+    assert classify_copy_in_layout(bucket) == g["layout_kind"]
+    assert bucket.world_size == len(g["shard_sizes"]) and bucket.max_shard_size == max(g["shard_sizes"]) and bucket.has_grads
+    # argument errors are raised before any device work (reference: grad_bucket.py:77-96)
+    n = bucket.world_size * bucket.max_shard_size
+    with pytest.raises(ValueError, match="1D"):
+        fill_reduce_scatter_input(bucket, torch.empty(1, n))
+    with pytest.raises(ValueError, match="expected"):
+        fill_reduce_scatter_input(bucket, torch.empty(n + 1))
+    with pytest.raises(ValueError, match="backend must be"):
+        fill_reduce_scatter_input(bucket, torch.empty(n), backend="nope")
+    if g["layout_kind"] != "flat_contiguous":
+        with pytest.raises(ValueError, match="flat bucket layout"):
+            fill_reduce_scatter_input(bucket, torch.empty(n), backend="flat_cat")
+    if g["layout_kind"] != "fsdp2_chunk":
+        with pytest.raises(ValueError, match="FSDP2-style"):
+            fill_reduce_scatter_input(bucket, torch.empty(n), backend="chunk_cat")
+    with pytest.raises(ValueError, match="at least one rank"):
+        fill_reduce_scatter_input(MatrixGradBucket((), 0, (), ()), torch.empty(0))
+
+
+def test_closed_form_plans():
+    specs = param_specs([("a", (4, 6)), ("b", (8,))])
+    plan = fsdp2_chunk_plan(specs, 2)
+    assert plan.shard_sizes == (16, 16)
+    assert plan.rank_segments[1] == (LayoutSegment(12, 24, 0), LayoutSegment(28, 32, 12))
+    with pytest.raises(ValueError, match="divisible"):
+        fsdp2_chunk_plan(param_specs([("a", (3,))]), 2)
+    plan = block_grid_plan(specs, (2, 2))
+    validate_shard_plan(plan)
+    assert plan.shard_sizes == (8, 8, 8, 8)
+    assert plan.rank_segments[3][:2] == (LayoutSegment(15, 18, 0), LayoutSegment(21, 24, 3))
+    assert plan.rank_segments[3][2] == LayoutSegment(30, 32, 6)
+    owner = whole_param_owner_plan(specs, 2, [1, 0])
+    assert owner.shard_sizes == (8, 24) and owner.rank_segments[1] == (LayoutSegment(0, 24, 0),)
+    assert rank_major_owner_order(specs, 2, [1, 0]) == [1, 0]
+    assert contiguous_even_plan(7, 3).shard_sizes == (3, 2, 2)
+    for w in (MLP_W2, HIDDEN2048_W4):
+        validate_shard_plan(w.plan())
+    assert MLP_W2.plan().shard_sizes == (131456, 131456)
+    assert HIDDEN2048_W4.total_numel == 50335744 and HIDDEN4096_W4_BLOCK.total_numel == 202383360
+
+
+def test_merge_runs_builds_strided_blocks():
+    # R/2 row segments of C/2 elements at source pitch C, destination pitch C/2 -> one 2-D run
+    rows, cols = 6, 8
+    src = [r * cols + 4 for r in range(3, 6)]
+    dst = [100 + k * 4 for k in range(3)]
+    merged = merge_runs(make_runs(src, dst, [4, 4, 4]))
+    assert merged.shape[0] == 1
+    run = merged[0]
+    assert (run["rows"], run["row_len"], run["src_stride"], run["dst_stride"], run["src_off"], run["dst_off"]) == (3, 4, 8, 4, 28, 100)
+    # back-to-back on both sides -> one longer segment; a break in the pitch starts a new run
+    assert merge_runs(make_runs([0, 4, 8], [0, 4, 8], [4, 4, 4]))[0]["row_len"] == 12
+    merged = merge_runs(make_runs([0, 8, 16, 40], [0, 4, 8, 12], [4, 4, 4, 4]))
+    assert [int(r["rows"]) for r in merged] == [3, 1]
+    # different sources never merge
+    runs = make_runs([0, 4], [0, 4], [4, 4])
+    runs["src_id"] = [0, 1]
+    assert merge_runs(runs).shape[0] == 2
+    assert merge_runs(make_runs([], [], [])).shape[0] == 0
+
+
+def test_fill_runs_cover_exactly_the_gaps():
+    fills = fill_runs_for_gaps(make_runs([0, 0], [2, 8], [3, 2]), 12)
+    assert [(int(f["dst_off"]), int(f["row_len"]), int(f["src_id"])) for f in fills] == [(0, 2, -1), (5, 3, -1), (10, 2, -1)]
+    assert fill_runs_for_gaps(make_runs([0], [0], [12]), 12).shape[0] == 0
+    with pytest.raises(ValueError, match="overlap"):
+        fill_runs_for_gaps(make_runs([0, 0], [0, 2], [3, 3]), 12)
+
+
+def test_grad_fill_runs_match_the_oracle_on_random_layouts():
+    import random
+
+    from tests.conftest import params_from_pairs
+    from tests.test_oracle_copy import random_plan
+
+    rng = random.Random(3)
+    for _ in range(30):
+        sizes = [rng.randint(1, 40) for _ in range(rng.randint(1, 6))]
+        params = params_from_pairs([(f"p{i}", n) for i, n in enumerate(sizes)])
+        total, world = sum(sizes), rng.randint(1, 4)
+        plan = random_plan(rng, total, world) if total > 1 else contiguous_even_plan(total, world)
+        max_shard = plan.max_shard_size
+        runs = grad_fill_runs(params, plan.rank_segments, max_shard)
+        grads = [torch.arange(n, dtype=torch.float32) + 100 * (i + 1) for i, n in enumerate(sizes)]
+        have = torch.zeros(world * max_shard)
+        for run in runs:
+            s, d, n = int(run["src_off"]), int(run["dst_off"]), int(run["row_len"])
+            have[d : d + n] = grads[int(run["src_id"])][s : s + n]
+        want = torch.full((world * max_shard,), -1.0)
+        O.fill_reduce_scatter_input(params, grads, plan.shard_sizes, plan.rank_segments, total, want)
+        assert torch.equal(have, want)
