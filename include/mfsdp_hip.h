@@ -137,7 +137,7 @@ int mfsdp_segment_program_run(mfsdp_segment_program* program, const void* const*
                               void* dst, void* stream);
 
 /* Launch tuning for experiments: blocks per CU of the persistent copy grid
- * (0 = library default), non-temporal load/store hints (0/1, -1 = default) and
+ * (0 = library default), non-temporal hints (0 none, 1 loads and stores, 2 loads only, 3 stores only, -1 = default) and
  * 128-bit loads in flight per lane (4 or 8; applies to programs created afterwards). */
 void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll);
 

@@ -3,12 +3,12 @@
 // Both operands are K-contiguous (an "NT" product), which is what every Newton-Schulz product
 // reduces to once X and X^T are both kept: X X^T, A A^T (A symmetric) and B (X^T)^T.  A workgroup owns
 // a BM x BN tile of C; its waves each own a (BM/WM) x (BN/WN) sub-tile built from 32x32x16 bf16 MFMAs
-// with fp32 accumulators.  K is walked in slabs of 64: the slab of P and Q is staged in LDS as rows of
-// 128 bytes whose eight 16-byte chunks are XOR-swizzled with (row / 2) % 8: the LDS has 64 banks of 4
-// bytes, two rows span them once, so any 16 consecutive rows read at one logical chunk touch every bank
-// exactly once and the 128-bit fragment reads are bank-conflict free.  Two LDS stages: the next slab streams
-// from HBM straight into LDS (global_load ... lds, no register round trip) while the current one feeds
-// the MFMAs.
+// with fp32 accumulators.  K is walked in slabs of BK (64 or 32): the slab of P and Q is staged in LDS as
+// rows of BK bf16 whose 16-byte chunks are XOR-swizzled with the row index: the LDS has 64 banks of 4
+// bytes, 256 / (2 BK) rows span them once, so any 16 consecutive rows read at one logical chunk touch every
+// bank exactly once and the 128-bit fragment reads are bank-conflict free.  STAGES slabs are resident: the
+// next ones stream from HBM straight into LDS (global_load ... lds, no register round trip) while the
+// current one feeds the MFMAs.
 //
 // Tile scheduling.  Tiles are handed to workgroups so that the groups sharing an XCD (block ids
 // congruent mod 8) work on neighbouring tiles and reuse that XCD's L2.  When the tile count is not a
@@ -31,9 +31,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kBK = 64;            // K slab, bf16 elements (128 bytes per row)
-constexpr int kChunksPerRow = 8;   // 16-byte chunks per slab row
 constexpr int kXcds = 8;
+constexpr int kSlabK = 64;  // K granularity of the schedule (operands are padded to it); a slab is BK <= 64 wide
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   const __bf16 l = static_cast<__bf16>(lo);
@@ -74,7 +73,7 @@ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_
   *tn = in_group / rows;
 }
 
-template <int BM, int BN, int WM, int WN, bool DIRECT>
+template <int BM, int BN, int WM, int WN, int BK, int STAGES>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kThreads = WM * WN * 64;
@@ -83,10 +82,15 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kWaveN = BN / WN;
   constexpr int TM = kWaveM / 32;     // 32x32 MFMA tiles per wave
   constexpr int TN = kWaveN / 32;
-  constexpr int kPChunks = BM * kChunksPerRow / kThreads;  // 16-byte chunks of the P slab per thread
-  constexpr int kQChunks = BN * kChunksPerRow / kThreads;
-  static_assert(BM * kChunksPerRow % kThreads == 0 && BN * kChunksPerRow % kThreads == 0, "slab must divide over threads");
-  constexpr int kStageElems = (BM + BN) * kBK;
+  constexpr int kChunks = BK / 8;               // 16-byte chunks per slab row (row = BK bf16)
+  constexpr int kRowsPerSweep = 128 / BK;       // slab rows that together span the 64 LDS banks once (256 bytes)
+  constexpr int kRowsPerLoad = 512 / BK;        // slab rows one wave-level 1 KiB load fills
+  constexpr int kSteps = BK / 16;               // k16 MFMA steps per slab
+  constexpr int kLoadsP = BM / kRowsPerLoad / kWaves, kLoadsQ = BN / kRowsPerLoad / kWaves;
+  constexpr int kLoadsPerSlab = kLoadsP + kLoadsQ;  // direct-to-LDS loads one wave issues per slab
+  static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0, "slab must divide over the waves");
+  static_assert(kSteps % 2 == 0 && STAGES >= 2 && (STAGES - 1) * kLoadsPerSlab < 64, "pipeline shape");
+  constexpr int kStageElems = (BM + BN) * BK;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -108,7 +112,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   tile_coords<4>(logical, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
   const int row0 = tm * BM;
   const int col0 = tn * BN;
-  const int k_slabs_total = a.K / kBK;
+  const int k_slabs_total = a.K / BK;
   const int ks_begin = whole ? 0 : static_cast<int>(static_cast<int64_t>(k_slabs_total) * split / sched.splits);
   const int ks_end = whole ? k_slabs_total : static_cast<int>(static_cast<int64_t>(k_slabs_total) * (split + 1) / sched.splits);
 
@@ -120,7 +124,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   auto k0_of = [&](int i) {
     int slab = i + k_start;
     if (slab >= n_slabs) slab -= n_slabs;
-    return (ks_begin + slab) * kBK;
+    return (ks_begin + slab) * BK;
   };
 
   const int tid = threadIdx.x;
@@ -132,62 +136,28 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   const __bf16* __restrict__ P = static_cast<const __bf16*>(a.P) + static_cast<int64_t>(row0) * a.ldp;
   const __bf16* __restrict__ Q = static_cast<const __bf16*>(a.Q) + static_cast<int64_t>(col0) * a.ldq;
 
-  // ---- slab loaders.  Chunk c of a slab = row c / 8, 16-byte chunk c % 8, stored at chunk (c%8) ^ ((row/2)%8).
-  // Register-staged: thread t handles chunks i*kThreads + t.
-  u32x4 pre_p[DIRECT ? 1 : kPChunks], pre_q[DIRECT ? 1 : kQChunks];
-  auto fetch = [&](int k0) {
-    if constexpr (!DIRECT) {
-#pragma unroll
-      for (int i = 0; i < kPChunks; ++i) {
-        const int c = i * kThreads + tid;
-        pre_p[i] = *reinterpret_cast<const u32x4*>(P + static_cast<int64_t>(c >> 3) * a.ldp + k0 + (c & 7) * 8);
-      }
-#pragma unroll
-      for (int i = 0; i < kQChunks; ++i) {
-        const int c = i * kThreads + tid;
-        pre_q[i] = *reinterpret_cast<const u32x4*>(Q + static_cast<int64_t>(c >> 3) * a.ldq + k0 + (c & 7) * 8);
-      }
-    }
-  };
-  auto stash = [&](int stage) {
-    if constexpr (!DIRECT) {
-      __bf16* sp = smem + stage * kStageElems;
-      __bf16* sq = sp + BM * kBK;
-#pragma unroll
-      for (int i = 0; i < kPChunks; ++i) {
-        const int c = i * kThreads + tid;
-        const int r = c >> 3;
-        *reinterpret_cast<u32x4*>(sp + r * kBK + (((c & 7) ^ ((r >> 1) & 7)) << 3)) = pre_p[i];
-      }
-#pragma unroll
-      for (int i = 0; i < kQChunks; ++i) {
-        const int c = i * kThreads + tid;
-        const int r = c >> 3;
-        *reinterpret_cast<u32x4*>(sq + r * kBK + (((c & 7) ^ ((r >> 1) & 7)) << 3)) = pre_q[i];
-      }
-    }
-  };
-  // Direct to LDS: one wave-level load fills 1 KiB = 8 rows; lane l lands at row l/8, chunk position l%8 and
-  // therefore fetches the global chunk that the swizzle maps there.  Wave w takes the 8-row groups w, w + kWaves, ...
-  const int dl_row = lane >> 3;
+  // ---- slab loader.  A slab row holds BK bf16 = kChunks 16-byte chunks; chunk c of row r is stored at chunk
+  // position c ^ ((r / kRowsPerSweep) % kChunks).  One wave-level direct-to-LDS load fills 1 KiB = kRowsPerLoad
+  // rows: lane l lands at row l / kChunks, position l % kChunks, and therefore fetches the global chunk the
+  // swizzle maps there.  Wave w takes the row groups w, w + kWaves, ...
+  const int dl_row = lane / kChunks;
+  const int dl_pos = lane % kChunks;
   auto stream_in = [&](int k0, int stage) {
-    if constexpr (DIRECT) {
-      __bf16* sp = smem + stage * kStageElems;
-      __bf16* sq = sp + BM * kBK;
+    __bf16* sp = smem + stage * kStageElems;
+    __bf16* sq = sp + BM * BK;
 #pragma unroll
-      for (int i = 0; i < BM / 8 / kWaves; ++i) {
-        const int r0 = (i * kWaves + wave) * 8;
-        const int dl_chunk = (lane & 7) ^ (((r0 + dl_row) >> 1) & 7);
-        const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + dl_chunk * 8;
-        __builtin_amdgcn_global_load_lds(src, sp + r0 * kBK, 16, 0, 0);
-      }
+    for (int i = 0; i < kLoadsP; ++i) {
+      const int r0 = (i * kWaves + wave) * kRowsPerLoad;
+      const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
+      const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + chunk * 8;
+      __builtin_amdgcn_global_load_lds(src, sp + r0 * BK, 16, 0, 0);
+    }
 #pragma unroll
-      for (int i = 0; i < BN / 8 / kWaves; ++i) {
-        const int r0 = (i * kWaves + wave) * 8;
-        const int dl_chunk = (lane & 7) ^ (((r0 + dl_row) >> 1) & 7);
-        const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + dl_chunk * 8;
-        __builtin_amdgcn_global_load_lds(src, sq + r0 * kBK, 16, 0, 0);
-      }
+    for (int i = 0; i < kLoadsQ; ++i) {
+      const int r0 = (i * kWaves + wave) * kRowsPerLoad;
+      const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
+      const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + chunk * 8;
+      __builtin_amdgcn_global_load_lds(src, sq + r0 * BK, 16, 0, 0);
     }
   };
 
@@ -202,16 +172,16 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   const int frag_row = lane & 31;   // row of the 32-row MFMA operand this lane supplies
   const int frag_half = lane >> 5;  // which 8 of the 16 k values
 
-  // LDS offsets of this lane's fragment chunk for the four k16 steps of a slab (the row part of the
-  // swizzle only depends on frag_row, every 32-row block starts at a multiple of 16 rows)
-  const __bf16* frag_p = smem + (wave_m * kWaveM + frag_row) * kBK;
-  const __bf16* frag_q = smem + BM * kBK + (wave_n * kWaveN + frag_row) * kBK;
+  // LDS offsets of this lane's fragment chunk for the k16 steps of a slab (the row part of the swizzle only
+  // depends on frag_row, every 32-row block starts at a multiple of 16 rows)
+  const __bf16* frag_p = smem + (wave_m * kWaveM + frag_row) * BK;
+  const __bf16* frag_q = smem + BM * BK + (wave_n * kWaveN + frag_row) * BK;
   auto load_frags = [&](int stage, int kk, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
-    const int off = stage * kStageElems + (((kk * 2 + frag_half) ^ ((frag_row >> 1) & 7)) << 3);
+    const int off = stage * kStageElems + (((kk * 2 + frag_half) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 32 * kBK);
+    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 32 * BK);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 32 * kBK);
+    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 32 * BK);
   };
   auto multiply = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
 #pragma unroll
@@ -220,71 +190,58 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
   };
 
-  if constexpr (DIRECT) {
-    // Software pipeline.  Fragments are double buffered in registers: the six (TM + TN) 128-bit LDS reads of
-    // step kk+1 are issued before the MFMAs of step kk, so their latency hides behind TM*TN MFMAs.  The one
-    // barrier per slab sits before the slab's last k16 step: by then every wave has its last fragments of the
-    // current stage in registers (the stage can be refilled) and its share of the next stage has landed, so
-    // the first fragments of the next slab are fetched under the last MFMAs of this one.
-    bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-    if (n_slabs > 0) {
-      stream_in(k0_of(0), 0);
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's chunks of the first slab are in LDS
-      __syncthreads();
-      if (n_slabs > 1) stream_in(k0_of(1), 1);
-      load_frags(0, 0, fa0, fb0);
-    }
-    // The fragments a k16 step multiplies were requested one step earlier; waiting for them BEFORE the next
-    // step's reads are issued costs nothing and leaves those reads a whole step of MFMAs to complete.
-    constexpr int kWaitLds = 0xC07F;  // s_waitcnt lgkmcnt(0), vmcnt / expcnt fields at their maxima
-    for (int it = 0; it < n_slabs; ++it) {
-      const int stage = it & 1;
-      __builtin_amdgcn_s_waitcnt(kWaitLds);
-      __builtin_amdgcn_sched_barrier(0);
-      load_frags(stage, 1, fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_waitcnt(kWaitLds);
-      __builtin_amdgcn_sched_barrier(0);
-      load_frags(stage, 2, fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_waitcnt(kWaitLds);
-      __builtin_amdgcn_sched_barrier(0);
-      load_frags(stage, 3, fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): last fragments in registers, next stage landed
-      if (it + 1 < n_slabs) {
-        __syncthreads();
-        if (it + 2 < n_slabs && !(sched.debug & 1)) stream_in(k0_of(it + 2), stage);
-        load_frags(stage ^ 1, 0, fa0, fb0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  } else {
-    if (n_slabs > 0) {
-      fetch(k0_of(0));
-      stash(0);
-      __syncthreads();
-    }
-    for (int it = 0; it < n_slabs; ++it) {
-      const int stage = it & 1;
-      if (it + 1 < n_slabs) fetch(k0_of(it + 1));
+  // Software pipeline.  STAGES slabs are resident or in flight: the slab being multiplied and the next
+  // STAGES - 1, streamed HBM -> LDS while the MFMAs run.  Fragments are double buffered in registers: the
+  // TM + TN 128-bit LDS reads of step kk+1 are issued before the MFMAs of step kk (and waited for BEFORE the
+  // reads of step kk+2 are issued, which costs nothing), so their latency hides behind TM*TN MFMAs.  The one
+  // barrier per slab sits before the slab's last k16 step: by then every wave has its last fragments of the
+  // current stage in registers (the stage can be refilled with the slab STAGES ahead) and its share of the next
+  // slab has landed, so the next slab's first fragments are fetched under this slab's last MFMAs.
+  constexpr int kWaitLds = 0xC07F;  // s_waitcnt lgkmcnt(0), vmcnt / expcnt fields at their maxima
+  // s_waitcnt lgkmcnt(0) vmcnt(N): loads return in order, so this leaves the N most recent ones in flight
+  constexpr int kInFlight = (STAGES - 2) * kLoadsPerSlab;
+  constexpr int kWaitNextSlab = 0x0070 | (kInFlight & 0xF) | ((kInFlight >> 4) << 14);
+  bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  if (n_slabs > 0) {
 #pragma unroll
-      for (int kk = 0; kk < kBK / 16; ++kk) {
-        bf16x8 fa[TM], fb[TN];
-        load_frags(stage, kk, fa, fb);
-        multiply(fa, fb);
+    for (int sidx = 0; sidx < STAGES; ++sidx)
+      if (sidx < n_slabs) stream_in(k0_of(sidx), sidx);
+    if (n_slabs >= STAGES) __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 1) * kLoadsPerSlab) & 0xF) | ((((STAGES - 1) * kLoadsPerSlab) >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    load_frags(0, 0, fa0, fb0);
+  }
+  int stage = 0;
+  for (int it = 0; it < n_slabs; ++it) {
+    const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+#pragma unroll
+    for (int kk = 0; kk < kSteps; kk += 2) {
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      load_frags(stage, kk + 1, fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk + 2 < kSteps) {
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_sched_barrier(0);
+        load_frags(stage, kk + 2, fa0, fb0);
+      } else if (it + 1 < n_slabs) {
+        // last step of the slab: the slab after it must have landed; the STAGES - 2 younger ones may be in flight
+        // (near the end of the walk fewer are, then wait for everything)
+        if (it + STAGES <= n_slabs) __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
+        else __builtin_amdgcn_s_waitcnt(0x0070);
+        __syncthreads();
+        if (it + STAGES < n_slabs && !(sched.debug & 1)) stream_in(k0_of(it + STAGES), stage);
+        load_frags(next_stage, 0, fa0, fb0);
+      } else {
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
       }
-      if (it + 1 < n_slabs) stash(stage ^ 1);
-      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    stage = next_stage;
   }
 
   // ---- K pieces: park the fp32 partial tile (row-major BM x BN); the fix-up kernel sums the pieces and
@@ -299,7 +256,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = wave_m * kWaveM + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-          __builtin_nontemporal_store(acc[i][j][r], mine + row * BN + col);
+          mine[row * BN + col] = acc[i][j][r];
         }
       }
     return;
@@ -392,9 +349,17 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
   const int row = tm * BM + lrow;
   const int col = tn * BN + lcol;
   const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
+  // four loads in flight at a time; the sum itself stays in split order
   f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int s = 0; s < sched.splits; ++s)
-    sum += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN)));
+  int s = 0;
+  for (; s + 4 <= sched.splits; s += 4) {
+    f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s + u) * (BM * BN));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sum += v[u];
+  }
+  for (; s < sched.splits; ++s) sum += *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN));
   const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
   uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
@@ -425,14 +390,14 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
 
 GemmTuning g_tuning;
 
-template <int BM, int BN, int WM, int WN, bool DIRECT>
+template <int BM, int BN, int WM, int WN, int BK, int STAGES>
 int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, hipStream_t stream) {
   Schedule s{};
   s.tiles_m = a.M / BM;
   s.tiles_n = a.N / BN;
   const int tiles = a.symmetric ? s.tiles_m * (s.tiles_m + 1) / 2 : s.tiles_m * s.tiles_n;
   const int slots = device_cu_count() * blocks_per_cu;
-  const int k_slabs = a.K / kBK;
+  const int k_slabs = a.K / BK;
   s.full_tiles = tiles;
   s.splits = 1;
   s.partials = static_cast<float*>(scratch.partials);
@@ -450,10 +415,10 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, h
     }
   }
   const int blocks = s.full_tiles + (tiles - s.full_tiles) * s.splits;
-  constexpr size_t smem_loop = 2 * static_cast<size_t>(BM + BN) * kBK * sizeof(uint16_t);
+  constexpr size_t smem_loop = static_cast<size_t>(STAGES) * (BM + BN) * BK * sizeof(uint16_t);
   constexpr size_t smem_epilogue = static_cast<size_t>(BM > BN ? BM : BN) * ((BM > BN ? BM : BN) + 8) * sizeof(uint16_t);
   constexpr size_t smem = smem_loop > smem_epilogue ? smem_loop : smem_epilogue;
-  auto kernel = gemm_nt_kernel<BM, BN, WM, WN, DIRECT>;
+  auto kernel = gemm_nt_kernel<BM, BN, WM, WN, BK, STAGES>;
   static bool configured = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!configured) {
     MFSDP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -476,8 +441,8 @@ void set_gemm_tuning(const GemmTuning& t) { g_tuning = t; }
 GemmTuning get_gemm_tuning() { return g_tuning; }
 
 int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
-  if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kBK)
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kBK);
+  if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kSlabK)
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kSlabK);
   if (a.symmetric && a.M != a.N) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric product needs M == N");
   if (!a.P || !a.Q || !a.C) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: null operand");
   if (a.ldp < a.K || a.ldq < a.K || a.ldc < a.N || (a.D && a.ldd < a.N) || (a.CT && a.ldct < a.M))
@@ -488,14 +453,19 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
       (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
   const int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
-  const bool direct = g_tuning.direct_to_lds != 0;
   switch (variant) {
     case 2:  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
-      return direct ? launch<128, 128, 2, 2, true>(a, scratch, 2, stream) : launch<128, 128, 2, 2, false>(a, scratch, 2, stream);
+      return launch<128, 128, 2, 2, 64, 2>(a, scratch, 2, stream);
     case 3:  // 256x256 tile, 4 waves of 128x128
-      return direct ? launch<256, 256, 2, 2, true>(a, scratch, 1, stream) : launch<256, 256, 2, 2, false>(a, scratch, 1, stream);
-    default:  // 256x256 tile, 8 waves of 128x64
-      return direct ? launch<256, 256, 2, 4, true>(a, scratch, 1, stream) : launch<256, 256, 2, 4, false>(a, scratch, 1, stream);
+      return launch<256, 256, 2, 2, 64, 2>(a, scratch, 1, stream);
+    case 4:  // 256x256 tile, 8 waves, slabs of 32 four deep
+      return launch<256, 256, 2, 4, 32, 4>(a, scratch, 1, stream);
+    case 5:  // 256x256 tile, 8 waves, slabs of 32 five deep (all 160 KiB of LDS)
+      return launch<256, 256, 2, 4, 32, 5>(a, scratch, 1, stream);
+    case 6:  // 128x128 tile, slabs of 32 four deep, two workgroups per CU
+      return launch<128, 128, 2, 2, 32, 4>(a, scratch, 2, stream);
+    default:  // 256x256 tile, 8 waves of 128x64, slabs of 64 two deep
+      return launch<256, 256, 2, 4, 64, 2>(a, scratch, 1, stream);
   }
 }
 

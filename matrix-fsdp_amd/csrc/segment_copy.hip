@@ -154,7 +154,7 @@ __device__ __forceinline__ Words<DST_B> convert_group(const Words<SRC_B>& in) {
   return out;
 }
 
-template <int SRC_B, int DST_B, int U, bool NT>
+template <int SRC_B, int DST_B, int U, bool NT, bool NTS = NT>
 __global__ void __launch_bounds__(kBlockThreads)
 segment_program_kernel(SourceTable srcs, char* __restrict__ dst, const DevRun* __restrict__ runs,
                        const DevTile* __restrict__ tiles, uint32_t n_tiles) {
@@ -189,13 +189,14 @@ segment_program_kernel(SourceTable srcs, char* __restrict__ dst, const DevRun* _
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (live[u]) store_bytes<DST_B, NT>(dst + doff[u] * DST_B, convert_group<SRC_B, DST_B>(data[u]));
+      if (live[u]) store_bytes<DST_B, NTS>(dst + doff[u] * DST_B, convert_group<SRC_B, DST_B>(data[u]));
     }
   }
 }
 
 struct Tuning {
-  int blocks_per_cu = 8;
+  int blocks_per_cu = 2;        // persistent grid of the segment kernel: 2 workgroups (8 waves) per CU measured best
+  int linear_blocks_per_cu = 16;  // contiguous range copies / casts want more workgroups in flight
   int nontemporal = 1;
   int unroll = 4;
 };
@@ -335,15 +336,19 @@ int launch_one(const Compiled& c, const SourceTable& srcs, char* dst, hipStream_
   const uint32_t cap = static_cast<uint32_t>(cus) * static_cast<uint32_t>(std::max(1, g_tuning.blocks_per_cu));
   const dim3 grid(std::max(1u, std::min(want, cap)));
   const dim3 block(kBlockThreads);
-  const bool nt = g_tuning.nontemporal != 0;
-#define MFSDP_LAUNCH(U_, NT_)                                                                              \
-  hipLaunchKernelGGL((segment_program_kernel<SRC_B, DST_B, U_, NT_>), grid, block, 0, stream, srcs, dst, \
+  const int nt = g_tuning.nontemporal;  // 0 none, 1 loads and stores, 2 loads only, 3 stores only
+#define MFSDP_LAUNCH(U_, NTL_, NTS_)                                                                             \
+  hipLaunchKernelGGL((segment_program_kernel<SRC_B, DST_B, U_, NTL_, NTS_>), grid, block, 0, stream, srcs, dst, \
                      c.runs, c.tiles, c.n_tiles)
-  if (c.unroll == 8) {
-    if (nt) MFSDP_LAUNCH(8, true); else MFSDP_LAUNCH(8, false);
-  } else {
-    if (nt) MFSDP_LAUNCH(4, true); else MFSDP_LAUNCH(4, false);
+#define MFSDP_LAUNCH_NT(U_)                      \
+  switch (nt) {                                  \
+    case 0: MFSDP_LAUNCH(U_, false, false); break; \
+    case 2: MFSDP_LAUNCH(U_, true, false); break;  \
+    case 3: MFSDP_LAUNCH(U_, false, true); break;  \
+    default: MFSDP_LAUNCH(U_, true, true); break;  \
   }
+  if (c.unroll == 8) { MFSDP_LAUNCH_NT(8) } else { MFSDP_LAUNCH_NT(4) }
+#undef MFSDP_LAUNCH_NT
 #undef MFSDP_LAUNCH
   MFSDP_CHECK_LAUNCH("segment_program_kernel");
   return MFSDP_OK;
@@ -392,8 +397,8 @@ int setup_units(int convert, int elem_bytes, int* src_unit, int* dst_unit, int* 
 }  // namespace
 
 extern "C" void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll) {
-  g_tuning.blocks_per_cu = blocks_per_cu > 0 ? blocks_per_cu : 8;
-  g_tuning.nontemporal = nontemporal < 0 ? 1 : (nontemporal != 0);
+  g_tuning.blocks_per_cu = blocks_per_cu > 0 ? blocks_per_cu : 2;
+  g_tuning.nontemporal = (nontemporal < 0 || nontemporal > 3) ? 1 : nontemporal;
   g_tuning.unroll = unroll == 8 ? 8 : 4;
 }
 
@@ -623,7 +628,7 @@ int launch_linear(const char* src, char* dst, int64_t n_groups, hipStream_t stre
   constexpr int U = 4;
   const int64_t span = static_cast<int64_t>(kBlockThreads) * U;
   const int64_t want = (n_groups + span - 1) / span;
-  const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.blocks_per_cu);
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.linear_blocks_per_cu);
   const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, cap))));
   if (g_tuning.nontemporal)
     hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, true>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
