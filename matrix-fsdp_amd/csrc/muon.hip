@@ -92,6 +92,10 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     g.M = w.mp; g.N = w.np; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.np; g.ldc = w.np; g.ldct = w.mp;
     g.alpha = 1.0f; g.beta = a; g.symmetric = 0;
+    if (s + 1 == steps) {  // the last step only has to leave O in the parameter's orientation
+      if (w.tall) g.skip_c = 1;
+      else g.CT = nullptr;
+    }
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
   }
   const int fin = steps & 1;

@@ -58,27 +58,81 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
   return total;  // valid in thread 0
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// four consecutive elements at index 4*v (the caller guarantees the alignment)
+template <typename T>
+struct Quad;
+template <>
+struct Quad<float> {
+  static __device__ __forceinline__ void load(const float* p, int64_t v, float (&out)[4]) {
+    const f32x4 q = reinterpret_cast<const f32x4*>(p)[v];
+    out[0] = q.x; out[1] = q.y; out[2] = q.z; out[3] = q.w;
+  }
+  static __device__ __forceinline__ void store(float* p, int64_t v, const float (&in)[4]) {
+    const f32x4 q = {in[0], in[1], in[2], in[3]};
+    reinterpret_cast<f32x4*>(p)[v] = q;
+  }
+};
+template <>
+struct Quad<uint16_t> {
+  static __device__ __forceinline__ void load(const uint16_t* p, int64_t v, float (&out)[4]) {
+    const u32x2 q = reinterpret_cast<const u32x2*>(p)[v];
+    out[0] = __uint_as_float(q.x << 16); out[1] = __uint_as_float(q.x & 0xffff0000u);
+    out[2] = __uint_as_float(q.y << 16); out[3] = __uint_as_float(q.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, int64_t v, const float (&in)[4]) {
+    const u32x2 q = {static_cast<uint32_t>(f32_to_bf16(in[0])) | (static_cast<uint32_t>(f32_to_bf16(in[1])) << 16),
+                     static_cast<uint32_t>(f32_to_bf16(in[2])) | (static_cast<uint32_t>(f32_to_bf16(in[3])) << 16)};
+    reinterpret_cast<u32x2*>(p)[v] = q;
+  }
+};
+
 // MOMENTUM: buf <- lerp(buf, g, 1-mu); u = nesterov ? lerp(g, buf, mu) : buf.   !MOMENTUM: u = g.
 // xraw <- bf16(u); partials[block] = sum of bf16(u)^2 over the block's elements.
 template <typename T, bool MOMENTUM>
+__device__ __forceinline__ float momentum_one(float g, float b_old, float momentum, float one_minus_momentum, int nesterov,
+                                              float* b_new, uint16_t* xb) {
+  float u = g;
+  if constexpr (MOMENTUM) {
+    const float b = Elem<T>::round(lerp_aten(b_old, g, one_minus_momentum));
+    *b_new = b;
+    u = nesterov ? Elem<T>::round(lerp_aten(g, b, momentum)) : b;
+  }
+  *xb = f32_to_bf16(u);
+  const float xf = bf16_to_f32(*xb);
+  return xf * xf;
+}
+
+// n_quads groups of four elements are processed with 128-bit (fp32) / 64-bit (bf16) accesses, the rest one by one.
+template <typename T, bool MOMENTUM>
 __global__ void __launch_bounds__(kThreads)
 momentum_kernel(const T* __restrict__ grad, T* __restrict__ buf, uint16_t* __restrict__ xraw, float* __restrict__ partials,
-                int64_t numel, float momentum, float one_minus_momentum, int nesterov) {
+                int64_t numel, int64_t n_quads, float momentum, float one_minus_momentum, int nesterov) {
   __shared__ float lds[kThreads / 64];
   float sumsq = 0.0f;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < numel; i += stride) {
-    const float g = Elem<T>::load(grad, i);
-    float u = g;
-    if constexpr (MOMENTUM) {
-      const float b = Elem<T>::round(lerp_aten(Elem<T>::load(buf, i), g, one_minus_momentum));
-      Elem<T>::store(buf, i, b);
-      u = nesterov ? Elem<T>::round(lerp_aten(g, b, momentum)) : b;
-    }
-    const uint16_t xb = f32_to_bf16(u);
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  for (int64_t v = first; v < n_quads; v += stride) {
+    float g[4], b[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bn[4];
+    Quad<T>::load(grad, v, g);
+    if constexpr (MOMENTUM) Quad<T>::load(buf, v, b);
+    uint16_t xb[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sumsq += momentum_one<T, MOMENTUM>(g[e], b[e], momentum, one_minus_momentum, nesterov, &bn[e], &xb[e]);
+    if constexpr (MOMENTUM) Quad<T>::store(buf, v, bn);
+    const u32x2 packed = {static_cast<uint32_t>(xb[0]) | (static_cast<uint32_t>(xb[1]) << 16),
+                          static_cast<uint32_t>(xb[2]) | (static_cast<uint32_t>(xb[3]) << 16)};
+    reinterpret_cast<u32x2*>(xraw)[v] = packed;
+  }
+  for (int64_t i = n_quads * 4 + first; i < numel; i += stride) {
+    float bn = 0.0f;
+    uint16_t xb;
+    sumsq += momentum_one<T, MOMENTUM>(Elem<T>::load(grad, i), MOMENTUM ? Elem<T>::load(buf, i) : 0.0f, momentum, one_minus_momentum,
+                                       nesterov, &bn, &xb);
+    if constexpr (MOMENTUM) Elem<T>::store(buf, i, bn);
     xraw[i] = xb;
-    const float xf = bf16_to_f32(xb);
-    sumsq += xf * xf;
   }
   const float total = block_sum(sumsq, lds);
   if (threadIdx.x == 0) partials[blockIdx.x] = total;
@@ -106,38 +160,67 @@ norm_kernel(const float* __restrict__ partials, int n_partials, float eps, float
 // 64 x 64 tile of the zero-padded outputs per block:
 //   same [r][c]  = bf16(x[r][c] / norm)   (rows_pad x cols_pad, ld = cols_pad)
 //   trans[c][r]  = same[r][c]             (cols_pad x rows_pad, ld = rows_pad)
-// with x = 0 outside rows x cols.
+// with x = 0 outside rows x cols.  Every thread handles groups of four consecutive elements: 64-bit stores on
+// both outputs (the padded buffers are 256-element aligned); the input is read 64 bits at a time when quads is set.
 __global__ void __launch_bounds__(kThreads)
-scale_transpose_kernel(const uint16_t* __restrict__ xraw, int rows, int cols, const float* __restrict__ scalars,
+scale_transpose_kernel(const uint16_t* __restrict__ xraw, int rows, int cols, int quads, const float* __restrict__ scalars,
                        uint16_t* __restrict__ same, uint16_t* __restrict__ trans, int rows_pad, int cols_pad) {
-  __shared__ uint16_t tile[64][66];
+  __shared__ uint16_t tile[64][68];
   const float norm = scalars[0];
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
-    const int lr = e >> 6, lc = e & 63;
+  for (int e = threadIdx.x; e < 64 * 16; e += kThreads) {
+    const int lr = e >> 4, lc = (e & 15) * 4;
     const int r = r0 + lr, c = c0 + lc;
-    uint16_t v = 0;
-    if (r < rows && c < cols) v = f32_to_bf16(__fdiv_rn(bf16_to_f32(xraw[static_cast<int64_t>(r) * cols + c]), norm));
-    tile[lr][lc] = v;
-    same[static_cast<int64_t>(r) * cols_pad + c] = v;
+    uint16_t raw[4] = {0, 0, 0, 0};
+    if (r < rows) {
+      if (quads && c + 3 < cols) {
+        const u32x2 q = *reinterpret_cast<const u32x2*>(xraw + static_cast<int64_t>(r) * cols + c);
+        raw[0] = static_cast<uint16_t>(q.x); raw[1] = static_cast<uint16_t>(q.x >> 16);
+        raw[2] = static_cast<uint16_t>(q.y); raw[3] = static_cast<uint16_t>(q.y >> 16);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (c + k < cols) raw[k] = xraw[static_cast<int64_t>(r) * cols + c + k];
+      }
+    }
+    uint16_t v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[k] = (r < rows && c + k < cols) ? f32_to_bf16(__fdiv_rn(bf16_to_f32(raw[k]), norm)) : static_cast<uint16_t>(0);
+      tile[lr][lc + k] = v[k];
+    }
+    const u32x2 packed = {static_cast<uint32_t>(v[0]) | (static_cast<uint32_t>(v[1]) << 16),
+                          static_cast<uint32_t>(v[2]) | (static_cast<uint32_t>(v[3]) << 16)};
+    *reinterpret_cast<u32x2*>(same + static_cast<int64_t>(r) * cols_pad + c) = packed;
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < 64 * 64; e += kThreads) {
-    const int lc = e >> 6, lr = e & 63;  // consecutive threads walk down a column of the tile = along a row of trans
-    trans[static_cast<int64_t>(c0 + lc) * rows_pad + r0 + lr] = tile[lr][lc];
+  for (int e = threadIdx.x; e < 64 * 16; e += kThreads) {
+    const int lc = e >> 4, lr = (e & 15) * 4;  // a row of trans = a column of the tile, four rows of the tile at a time
+    const u32x2 packed = {static_cast<uint32_t>(tile[lr][lc]) | (static_cast<uint32_t>(tile[lr + 1][lc]) << 16),
+                          static_cast<uint32_t>(tile[lr + 2][lc]) | (static_cast<uint32_t>(tile[lr + 3][lc]) << 16)};
+    *reinterpret_cast<u32x2*>(trans + static_cast<int64_t>(c0 + lc) * rows_pad + r0 + lr) = packed;
   }
 }
 
-// p <- round(round(p * decay) + neg_lr * o) over rows x cols, o read with leading dimension ldo.
+// p <- round(round(p * decay) + neg_lr * o) over rows x cols, o read with leading dimension ldo.  col_quads
+// groups of four columns per row use vector accesses (the caller guarantees their alignment).
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
-apply_kernel(T* __restrict__ param, const uint16_t* __restrict__ ortho, int rows, int cols, int ldo, float decay, float neg_lr) {
+apply_kernel(T* __restrict__ param, const uint16_t* __restrict__ ortho, int rows, int cols, int ldo, int col_quads, float decay,
+             float neg_lr) {
   for (int r = blockIdx.y; r < rows; r += gridDim.y) {
-    for (int c = blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads) {
-      const int64_t i = static_cast<int64_t>(r) * cols + c;
-      const float p = Elem<T>::round(Elem<T>::load(param, i) * decay);
-      Elem<T>::store(param, i, p + neg_lr * bf16_to_f32(ortho[static_cast<int64_t>(r) * ldo + c]));
+    T* prow = param + static_cast<int64_t>(r) * cols;
+    const uint16_t* orow = ortho + static_cast<int64_t>(r) * ldo;
+    for (int v = blockIdx.x * kThreads + threadIdx.x; v < col_quads; v += gridDim.x * kThreads) {
+      float p[4], o[4];
+      Quad<T>::load(prow, v, p);
+      Quad<uint16_t>::load(orow, v, o);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) p[e] = Elem<T>::round(p[e] * decay) + neg_lr * o[e];
+      Quad<T>::store(prow, v, p);
     }
+    for (int c = col_quads * 4 + blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads)
+      Elem<T>::store(prow, c, Elem<T>::round(Elem<T>::load(prow, c) * decay) + neg_lr * bf16_to_f32(orow[c]));
   }
 }
 
@@ -162,16 +245,20 @@ int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, float m
   // the scalar the reference hands to lerp_ is the Python double 1 - momentum
   const float one_minus = static_cast<float>(1.0 - static_cast<double>(momentum));
   auto x = static_cast<uint16_t*>(xraw);
+  const uintptr_t need = dtype == MFSDP_F32 ? 16 : 8;  // alignment of a group of four elements
+  const bool aligned = reinterpret_cast<uintptr_t>(grad) % need == 0 && (!with_momentum || reinterpret_cast<uintptr_t>(buf) % need == 0) &&
+                       reinterpret_cast<uintptr_t>(xraw) % 8 == 0;
+  const int64_t n_quads = aligned ? numel / 4 : 0;
   if (dtype == MFSDP_F32) {
     auto g = static_cast<const float*>(grad);
     auto b = static_cast<float*>(buf);
-    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<float, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
-    else hipLaunchKernelGGL((momentum_kernel<float, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<float, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<float, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
   } else {
     auto g = static_cast<const uint16_t*>(grad);
     auto b = static_cast<uint16_t*>(buf);
-    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<uint16_t, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
-    else hipLaunchKernelGGL((momentum_kernel<uint16_t, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, momentum, one_minus, nesterov);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<uint16_t, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<uint16_t, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
   }
   MFSDP_CHECK_LAUNCH("momentum_kernel");
   return MFSDP_OK;
@@ -186,7 +273,8 @@ int muon_norm(const float* partials, int n_partials, float eps, float* scalars, 
 int muon_scale_transpose(const void* xraw, int rows, int cols, const float* scalars, void* same, void* trans, int rows_pad,
                          int cols_pad, hipStream_t stream) {
   const dim3 grid(cols_pad / 64, rows_pad / 64);
-  hipLaunchKernelGGL(scale_transpose_kernel, grid, dim3(kThreads), 0, stream, static_cast<const uint16_t*>(xraw), rows, cols,
+  const int quads = (cols % 4 == 0 && reinterpret_cast<uintptr_t>(xraw) % 8 == 0) ? 1 : 0;
+  hipLaunchKernelGGL(scale_transpose_kernel, grid, dim3(kThreads), 0, stream, static_cast<const uint16_t*>(xraw), rows, cols, quads,
                      scalars, static_cast<uint16_t*>(same), static_cast<uint16_t*>(trans), rows_pad, cols_pad);
   MFSDP_CHECK_LAUNCH("scale_transpose_kernel");
   return MFSDP_OK;
@@ -194,12 +282,16 @@ int muon_scale_transpose(const void* xraw, int rows, int cols, const float* scal
 
 int muon_apply(void* param, int dtype, const void* ortho, int rows, int cols, int ldo, float decay, float neg_lr,
                hipStream_t stream) {
-  const dim3 grid(std::max(1, std::min((cols + kThreads - 1) / kThreads, 64)), std::min(rows, 65535));
   auto o = static_cast<const uint16_t*>(ortho);
+  const uintptr_t need = dtype == MFSDP_F32 ? 16 : 8;
+  const bool aligned = cols % 4 == 0 && ldo % 4 == 0 && reinterpret_cast<uintptr_t>(param) % need == 0 && reinterpret_cast<uintptr_t>(ortho) % 8 == 0;
+  const int col_quads = aligned ? cols / 4 : 0;
+  const int per_row = aligned ? col_quads : cols;
+  const dim3 grid(std::max(1, std::min((per_row + kThreads - 1) / kThreads, 64)), std::min(rows, 65535));
   if (dtype == MFSDP_F32)
-    hipLaunchKernelGGL((apply_kernel<float>), grid, dim3(kThreads), 0, stream, static_cast<float*>(param), o, rows, cols, ldo, decay, neg_lr);
+    hipLaunchKernelGGL((apply_kernel<float>), grid, dim3(kThreads), 0, stream, static_cast<float*>(param), o, rows, cols, ldo, col_quads, decay, neg_lr);
   else
-    hipLaunchKernelGGL((apply_kernel<uint16_t>), grid, dim3(kThreads), 0, stream, static_cast<uint16_t*>(param), o, rows, cols, ldo, decay, neg_lr);
+    hipLaunchKernelGGL((apply_kernel<uint16_t>), grid, dim3(kThreads), 0, stream, static_cast<uint16_t*>(param), o, rows, cols, ldo, col_quads, decay, neg_lr);
   MFSDP_CHECK_LAUNCH("apply_kernel");
   return MFSDP_OK;
 }

@@ -11,7 +11,7 @@ namespace mfsdp {
 //   P: M x K row-major (ldp), Q: N x K row-major (ldq), D / C: M x N row-major (ldd / ldc).
 //   M, N multiples of 256 and K a multiple of 64 (callers zero-pad their operands).
 //   D may be null (beta ignored).  CT, when non-null, also receives the transpose: CT[n][m] = C[m][n]
-//   (ldct).  symmetric: P*Q^T is known to be symmetric (M == N); only tiles on or below the diagonal are
+//   (ldct); with skip_c only CT is written.  symmetric: P*Q^T is known to be symmetric (M == N); only tiles on or below the diagonal are
 //   computed and each off-diagonal tile is also written mirrored into C.
 struct GemmNtArgs {
   const void* P;
@@ -23,6 +23,7 @@ struct GemmNtArgs {
   int ldp, ldq, ldd, ldc, ldct;
   float alpha, beta;
   int symmetric;
+  int skip_c;  // general product with CT set: write only the transposed output
 };
 
 // Device scratch for the K-split pieces of the last partial round of tiles (fp32 partial tiles).

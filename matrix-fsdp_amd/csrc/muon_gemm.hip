@@ -302,22 +302,25 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
         acc[i][j][r] = v;
       }
   if (D != nullptr) __syncthreads();  // the D tile has been consumed
+  if (!a.skip_c) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32] =
-            __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
-  __syncthreads();
-  for (int c = tid; c < BM * kRowChunks; c += kThreads) {
-    const int r = c / kRowChunks, cc = c - r * kRowChunks;
-    *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(row0 + r) * a.ldc + col0 + cc * 8) =
-        *reinterpret_cast<const u32x4*>(stage_c + r * kLdS + cc * 8);
+        for (int r = 0; r < 16; ++r)
+          stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32] =
+              __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
+    __syncthreads();
+    for (int c = tid; c < BM * kRowChunks; c += kThreads) {
+      const int r = c / kRowChunks, cc = c - r * kRowChunks;
+      *reinterpret_cast<u32x4*>(C + static_cast<int64_t>(row0 + r) * a.ldc + col0 + cc * 8) =
+          *reinterpret_cast<const u32x4*>(stage_c + r * kLdS + cc * 8);
+    }
+    if (CT == nullptr) return;
+    __syncthreads();
   }
   if (CT == nullptr) return;
-  __syncthreads();
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -379,7 +382,7 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
   const uint32_t lo = pack_bf16x2(v[0], v[1]);
   const uint32_t hi = pack_bf16x2(v[2], v[3]);
   u32x2 packed = {lo, hi};
-  *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
+  if (!a.skip_c) *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
   if (CT != nullptr) {
     CT[static_cast<int64_t>(col) * ldct + row] = static_cast<uint16_t>(lo);
     CT[static_cast<int64_t>(col + 1) * ldct + row] = static_cast<uint16_t>(lo >> 16);
@@ -444,6 +447,7 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kSlabK)
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kSlabK);
   if (a.symmetric && a.M != a.N) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric product needs M == N");
+  if (a.skip_c && (a.symmetric || !a.CT)) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: skip_c needs a transposed output and a general product");
   if (!a.P || !a.Q || !a.C) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: null operand");
   if (a.ldp < a.K || a.ldq < a.K || a.ldc < a.N || (a.D && a.ldd < a.N) || (a.CT && a.ldct < a.M))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: leading dimension smaller than the row length");
