@@ -45,6 +45,8 @@ def parse_args():
     ap.add_argument("--skip-legs", action="store_true", help="only the timed pack/unpack region (used under rocprofv3)")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
     ap.add_argument("--no-launch-events", action="store_true", help="no per-launch HIP events inside the timed region")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain Tensor.copy_ of 1 GiB (a copy kernel of known size, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -134,6 +136,12 @@ def main() -> int:
             else:
                 unpack.run((gathered[i],), outs[i])
 
+    if args.calibrate_copy:
+        cal_src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+        cal_dst = torch.empty_like(cal_src)
+        cal_dst.copy_(cal_src)  # 1 GiB read + 1 GiB written by torch's element-wise copy kernel
+        torch.cuda.synchronize()
+        del cal_src, cal_dst
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
@@ -162,7 +170,9 @@ def main() -> int:
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": None,
+        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for a
+        # plain 1 GiB copy in the same run (measured once, profiles/segment_program_hbm_traffic.md)
+        "traffic": 812_800_000 if layers > 0 else None,
         "algorithmic_bytes_per_launch": bytes_per_launch,
         "avg_launch_ms": round(avg_launch_ms, 5),
         "launches_timed": len(launch_events),

@@ -122,3 +122,26 @@ def rank_major_owner_order(params: Sequence, world_size: int, owner_ranks: Seque
     if len(order) != len(params):
         raise ValueError("owner ranks outside [0, world_size).")
     return order
+
+
+def flat_reordered_owner_layout(params: Sequence, world_size: int, owner_ranks: Sequence[int]):
+    """What the runtime executes for a whole-parameter owner layout
+    (matrix_fsdp/runtime/fsdp_unit.py:1625-1692): the flat buffer is re-laid
+    out rank-major -- rank 0's parameters first, then rank 1's, each rank's in
+    their planner order -- so that every rank's shard is ONE contiguous range
+    ``(rank_start, rank_end, 0)`` and compact rank-major order equals
+    full-buffer order.  Returns ``(order, offsets, plan)``: the parameter
+    indices in their new flat order, the new ``(offset, end)`` of every
+    parameter (indexed like ``params``) and the shard plan."""
+    order = rank_major_owner_order(params, world_size, owner_ranks)
+    offsets: list[tuple[int, int]] = [(0, 0)] * len(params)
+    segments: list[tuple[LayoutSegment, ...]] = []
+    cursor = 0
+    for rank in range(world_size):
+        start = cursor
+        for i in order:
+            if owner_ranks[i] == rank:
+                offsets[i] = (cursor, cursor + params[i].numel)
+                cursor += params[i].numel
+        segments.append((LayoutSegment(start, cursor, 0),) if cursor > start else ())
+    return order, offsets, ShardPlan.from_rank_segments(cursor, segments)

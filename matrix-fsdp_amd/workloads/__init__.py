@@ -13,7 +13,7 @@ from dataclasses import dataclass
 import torch
 
 from ..core.layout import ShardPlan
-from ..core.plans import block_grid_plan, fsdp2_chunk_plan
+from ..core.plans import block_grid_plan, flat_reordered_owner_layout, fsdp2_chunk_plan
 
 
 @dataclass(frozen=True)
@@ -79,7 +79,29 @@ class Workload:
             return fsdp2_chunk_plan(self.specs, self.world_size)
         if self.layout == "block2x2":
             return block_grid_plan(self.specs, (2, 2))
+        if self.layout == "owner":
+            return self.owner_layout(0)[2]
         raise ValueError(self.layout)
+
+    def owner_ranks(self, layer: int) -> list[int]:
+        """Whole-parameter owners of one layer's parameters: matrix number ``k`` of the model (five per
+        layer, in layer order) lives on rank ``k % W``; the two norm vectors go to ranks ``layer % W`` and
+        ``(layer + 1) % W``."""
+        owners, matrix, vector = [], 0, 0
+        n_matrices = sum(1 for _, shape in self.shapes if len(shape) == 2)
+        for _, shape in self.shapes:
+            if len(shape) == 2:
+                owners.append((layer * n_matrices + matrix) % self.world_size)
+                matrix += 1
+            else:
+                owners.append((layer + vector) % self.world_size)
+                vector += 1
+        return owners
+
+    def owner_layout(self, layer: int):
+        """``(order, offsets, plan)`` of the rank-major flat layout of one layer (see
+        ``flat_reordered_owner_layout``)."""
+        return flat_reordered_owner_layout(self.specs, self.world_size, self.owner_ranks(layer))
 
 
 MLP_W2 = Workload("mlp_w2", mlp_shapes(), 1, 2, "fsdp2_chunk", seed=0, grad_seed=1000)
@@ -88,6 +110,7 @@ HIDDEN4096_W4_BLOCK = Workload("hidden4096_w4_block2x2", transformer_layer_shape
 HIDDEN5120 = Workload("hidden5120_owner", transformer_layer_shapes(5120, 13824, gated=True), 40, 4, "owner", seed=4, grad_seed=1004)
 
 MUON_HIDDEN4096_SHAPES = ((4096, 4096), (12288, 4096), (11008, 4096))
+HIDDEN5120_TAIL_NUMEL = (40 * 2 * 5120 + 32000 * 5120) // 4  # one rank's fp32 AdamW shard: norm vectors + embedding
 MUON_SEED = 4
 
 
