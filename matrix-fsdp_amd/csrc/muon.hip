@@ -169,6 +169,6 @@ extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant
   if (direct_to_lds > 0) t.direct_to_lds = direct_to_lds == 1;
   if (split_remainder > 0) t.split_remainder = split_remainder == 1;
   if (max_splits > 0) t.max_splits = max_splits;
-  if (stagger >= 0) { t.stagger = stagger & 0xffff; t.debug = stagger >> 16; }
+  if (stagger >= 0) t.stagger = stagger;
   set_gemm_tuning(t);
 }

@@ -41,7 +41,6 @@ struct GemmTuning {
   int split_remainder = 1;    // split the tiles of the last partial round along K
   int max_splits = 16;
   int stagger = 0;            // K-walk start offset (slabs) between consecutive tiles; 0 = none
-  int debug = 0;              // experiments only (wrong results): bit 0 = no slab streaming after the first two
 };
 void set_gemm_tuning(const GemmTuning& tuning);
 GemmTuning get_gemm_tuning();

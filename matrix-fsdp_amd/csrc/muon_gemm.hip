@@ -48,7 +48,6 @@ struct Schedule {
   int splits;       // K pieces per remaining tile (block ids from full_tiles on); 1 when nothing remains
   float* partials;  // [remaining tiles][splits][BM][BN] fp32
   int stagger;      // tile t starts its K walk (t * stagger) slabs in and wraps around; 0 = every tile starts at slab 0
-  int debug;        // experiments only: bit 0 = skip the HBM -> LDS streaming after the first two slabs
 };
 
 // logical tile index -> (tm, tn)
@@ -232,7 +231,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
         if (it + STAGES <= n_slabs) __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
         else __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
-        if (it + STAGES < n_slabs && !(sched.debug & 1)) stream_in(k0_of(it + STAGES), stage);
+        if (it + STAGES < n_slabs) stream_in(k0_of(it + STAGES), stage);
         load_frags(next_stage, 0, fa0, fb0);
       } else {
         __builtin_amdgcn_s_waitcnt(kWaitLds);
@@ -262,7 +261,6 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     return;
   }
 
-  if (sched.debug & 2) return;  // experiments only: no epilogue
 
   // ---- epilogue, staged through LDS so that HBM only sees whole 16-byte-per-lane, row-contiguous accesses.
   // Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile: written
@@ -405,7 +403,6 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, h
   s.splits = 1;
   s.partials = static_cast<float*>(scratch.partials);
   s.stagger = g_tuning.stagger;
-  s.debug = g_tuning.debug;
   const int rem = tiles % slots;
   if (g_tuning.split_remainder && rem != 0 && scratch.partials != nullptr) {
     // fill the machine once more with pieces of the leftover tiles; cap the pieces per tile so that the summing stays short

@@ -1,0 +1,105 @@
+"""The mixed optimizer step of the whole-parameter owner layout, end to end on reduced shapes: gradient copy-in for
+the owner layout, Muon on the matrices rank 0 owns, fused AdamW on its fp32 tail shard, and pack / unpack of the
+rank-major flat buffers -- every stage against the CPU oracle (copies bit-exact, Muon within the stated tolerance),
+plus the full-size Newton-Schulz shapes of the hidden4096 model against the oracle."""
+import pytest
+import torch
+
+from matrix_fsdp_amd.kernels.segment_program import compact_owner_program, pack_program, unpack_program
+from matrix_fsdp_amd.optim import functional as F
+from matrix_fsdp_amd.workloads import ParamSpec, Workload, normal_flat, transformer_layer_shapes
+from oracle import copy_oracle as CO
+from oracle import optim_oracle as OO
+from tests.test_copy_gpu import assert_same_bits
+from tests.test_optim_gpu import max_err_over_scale, rel_fro
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MUON_TOL = 1e-2  # relative Frobenius error against torch.optim.Muon's arithmetic, the path's stated tolerance
+
+SMALL_OWNER = Workload("hidden192_owner", transformer_layer_shapes(192, 512, gated=True), 5, 4, "owner", seed=11, grad_seed=1011)
+
+
+def reordered_specs(w: Workload, layer: int):
+    order, offsets, plan = w.owner_layout(layer)
+    specs = [ParamSpec(s.fqn, s.shape, *offsets[i]) for i, s in enumerate(w.specs)]
+    return order, specs, plan
+
+
+@pytest.mark.parametrize("layer", range(SMALL_OWNER.layers))
+def test_owner_layout_pack_unpack_and_grad_copy_in(layer):
+    w = SMALL_OWNER
+    order, specs, plan = reordered_specs(w, layer)
+    assert CO.packed_rank_shards_are_full_tensor_order(plan)
+    assert len(set(plan.shard_sizes)) > 1  # uneven shards: the padded staging is exercised
+    full = normal_flat(plan.total_numel, 0.02, w.seed + layer, torch.bfloat16)
+    padded = torch.full((w.world_size * plan.max_shard_size,), 3, dtype=torch.bfloat16, device=DEV)
+    pack_program(plan, torch.bfloat16, device=DEV).run((full.to(DEV),), padded)
+    assert_same_bits(padded, CO.pack_to_padded(full, plan))
+    out = torch.full((plan.total_numel,), 5, dtype=torch.bfloat16, device=DEV)
+    unpack_program(plan, torch.bfloat16, device=DEV).run((padded,), out)
+    assert_same_bits(out, full)
+
+    # gradients of whole-parameter owners go to the reduce-scatter input at their packed offsets, cast to fp32
+    by_offset = sorted(specs, key=lambda s: s.offset)
+    grads = [normal_flat(s.numel, 1e-3, w.grad_seed + 16 * layer + k, torch.bfloat16) for k, s in enumerate(by_offset)]
+    expect = CO.fill_compact_owner_reduce_scatter_input(
+        by_offset, [g.float() for g in grads], plan.shard_sizes, plan.rank_segments, torch.full((sum(plan.shard_sizes),), -1.0)
+    )
+    offsets = [CO.packed_grad_offset_for_param(s, plan.shard_sizes, plan.rank_segments, compact=True) for s in by_offset]
+    assert offsets == [s.offset for s in by_offset]  # rank-major flat order: packed offset == flat offset
+    program = compact_owner_program(by_offset, offsets, sum(plan.shard_sizes), torch.bfloat16, torch.float32, device=DEV)
+    packed = torch.full((sum(plan.shard_sizes),), -1.0, device=DEV)
+    program.run([g.to(DEV) for g in grads], packed)
+    assert_same_bits(packed, expect)
+
+
+def test_rank0_mixed_update_over_all_layers():
+    w = SMALL_OWNER
+    ws = F.MuonWorkspace(DEV)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    owned = 0
+    tail = []
+    for layer in range(w.layers):
+        for i, (spec, owner) in enumerate(zip(w.specs, w.owner_ranks(layer))):
+            if owner != 0:
+                continue
+            seed = 100 * layer + i
+            if len(spec.shape) == 1:
+                tail.append(spec.numel)
+                continue
+            owned += 1
+            p = normal_flat(spec.numel, 0.02, seed, torch.float32).view(spec.shape)
+            g = normal_flat(spec.numel, 1e-3, seed + 50, torch.bfloat16).float().view(spec.shape)
+            buf = normal_flat(spec.numel, 1e-3, seed + 70, torch.float32).view(spec.shape)
+            p_dev, buf_dev = p.to(DEV), buf.to(DEV)
+            F.muon_step(p_dev, g.to(DEV), buf_dev, workspace=ws, **kw)
+            p_ref, buf_ref = p.clone(), buf.clone()
+            OO.muon_step(p_ref, g, buf_ref, **kw)
+            assert rel_fro(p_dev.cpu() - p, p_ref - p) < MUON_TOL, spec
+            assert torch.allclose(buf_dev.cpu(), buf_ref, rtol=1e-6, atol=1e-9)
+    assert owned == (w.layers * 5 + 3) // 4
+    # the tail: this rank's norm vectors and its quarter of a 1000 x 192 embedding, one flat fp32 shard
+    n = sum(tail) + 1000 * 192 // 4
+    p, g = normal_flat(n, 0.02, 7, torch.float32), normal_flat(n, 1e-3, 8, torch.bfloat16)
+    m, v = torch.zeros(n), torch.zeros(n)
+    dev = [t.to(DEV) for t in (p, g, m, v)]
+    for step in (1, 2, 3):
+        F.adamw_step(*dev, step, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+        OO.adamw_step(p, g.float(), m, v, step, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for have, want in zip((dev[0], dev[2], dev[3]), (p, m, v)):
+        assert max_err_over_scale(have, want) < 1e-6
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (4096, 11008)])
+def test_newton_schulz_full_size_against_oracle(shape):
+    """The bench shapes themselves (the wide one in its transposed, cheaper-for-the-CPU orientation is the same
+    arithmetic: both sides transpose tall inputs first)."""
+    torch.set_num_threads(16)
+    u = normal_flat(shape[0] * shape[1], 1e-3, 4, torch.float32).view(shape)
+    have = F.newton_schulz(u.to(DEV)).float().cpu()
+    want = OO.newton_schulz(u).float()
+    assert rel_fro(have, want) < MUON_TOL
+    # the bulk of the singular values was pushed into the band the quintic iteration converges to
+    s = torch.linalg.svdvals(have[:512].double() @ have[:512].double().T).sqrt()
+    assert float(s.max()) < 1.3 and float(s.median()) > 0.5
