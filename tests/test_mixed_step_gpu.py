@@ -94,12 +94,25 @@ def test_rank0_mixed_update_over_all_layers():
 @pytest.mark.parametrize("shape", [(4096, 4096), (4096, 11008)])
 def test_newton_schulz_full_size_against_oracle(shape):
     """The bench shapes themselves (the wide one in its transposed, cheaper-for-the-CPU orientation is the same
-    arithmetic: both sides transpose tall inputs first)."""
+    arithmetic: both sides transpose tall inputs first).
+
+    The bf16 iteration is chaotic at the last bit: two implementations with the same rounding points that differ
+    only in the order of their fp32 accumulations drift apart by about 10x per step (5e-6 after step one, 5e-3
+    after step five at 1024 x 2752 on the CPU), and at these sizes torch's CPU and GPU executions of the very same
+    ``_zeropower_via_newtonschulz`` are about 1e-2 apart.  So the tolerance is asserted against the optimizer the
+    reference instantiates, executed where the reference executes it (this GPU), and the CPU oracle is held to
+    the tolerance or to the distance torch's own GPU execution has from it, whichever is larger."""
+    from torch.optim._muon import _zeropower_via_newtonschulz
+
     torch.set_num_threads(16)
     u = normal_flat(shape[0] * shape[1], 1e-3, 4, torch.float32).view(shape)
     have = F.newton_schulz(u.to(DEV)).float().cpu()
+    torch_gpu = _zeropower_via_newtonschulz(u.to(DEV), OO.NS_COEFFICIENTS, 5, OO.NS_EPS).float().cpu()
     want = OO.newton_schulz(u).float()
-    assert rel_fro(have, want) < MUON_TOL
+    to_torch_gpu, to_oracle, torch_gpu_to_oracle = rel_fro(have, torch_gpu), rel_fro(have, want), rel_fro(torch_gpu, want)
+    print(f"newton_schulz {shape}: vs torch on this GPU {to_torch_gpu:.3e}, vs CPU oracle {to_oracle:.3e}, torch GPU vs CPU oracle {torch_gpu_to_oracle:.3e}")
+    assert to_torch_gpu < MUON_TOL
+    assert to_oracle < max(MUON_TOL, 1.1 * torch_gpu_to_oracle)
     # the bulk of the singular values was pushed into the band the quintic iteration converges to
     s = torch.linalg.svdvals(have[:512].double() @ have[:512].double().T).sqrt()
     assert float(s.max()) < 1.3 and float(s.median()) > 0.5
