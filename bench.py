@@ -44,6 +44,7 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=0, help="layer buffers of the hidden4096 workload (0 = all 32)")
     ap.add_argument("--skip-legs", action="store_true", help="only the timed pack/unpack region (used under rocprofv3)")
     ap.add_argument("--skip-mixed", action="store_true", help="skip the hidden5120 mixed-step leg")
+    ap.add_argument("--legs", default="rows,muon,adamw,mixed", help="comma list of the extra legs to run: rows (hidden2048 row split), muon, adamw, mixed")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
     ap.add_argument("--no-launch-events", action="store_true", help="no per-launch HIP events inside the timed region")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -204,7 +205,12 @@ def main() -> int:
     torch.cuda.empty_cache()
 
     legs = {}
-    if not args.skip_legs:
+    want = set() if args.skip_legs else {name for name in args.legs.split(",") if name}
+    if args.skip_mixed:
+        want.discard("mixed")
+    if "mixed" in want:
+        want |= {"muon", "adamw"}  # the mixed step reuses their set-up
+    if "rows" in want:
         # -------------------------------------------------------------- hidden2048 row split: pack / unpack / chunk-cat + cast
         w2 = HIDDEN2048_W4
         plan2 = w2.plan()
@@ -239,6 +245,7 @@ def main() -> int:
         del full2, gath2, out2, grads2, packed32
         torch.cuda.empty_cache()
 
+    if "muon" in want:
         # -------------------------------------------------------------- Muon on the hidden4096 matrices
         ws = F.MuonWorkspace(dev)
         genm = torch.Generator(device=dev).manual_seed(MUON_SEED)
@@ -287,6 +294,7 @@ def main() -> int:
         del mats
         torch.cuda.empty_cache()
 
+    if "adamw" in want:
         # -------------------------------------------------------------- fused AdamW on a flat fp32 shard
         n_adam = HIDDEN5120_TAIL_NUMEL
         pa, ga = torch.randn(n_adam, device=dev) * 0.02, torch.randn(n_adam, device=dev) * 1e-3
@@ -296,10 +304,11 @@ def main() -> int:
         del pa, ga, ma, va
         torch.cuda.empty_cache()
 
+    if "mixed" in want:
         # -------------------------------------------------------------- hidden5120 mixed step, rank 0 of a simulated world of 4:
         # pack + unpack of the 40 rank-major owner-layout layer buffers (uneven shards, padded staging), AdamW on the fp32
         # tail shard, Muon on the 50 matrices this rank owns
-        if not args.skip_mixed:
+        if True:
             w5 = HIDDEN5120
             progs = {}
             for k in range(w5.world_size):  # the owner pattern repeats every world_size layers
@@ -351,6 +360,7 @@ def main() -> int:
             }
             del mats5, pa, ga, ma, va
             torch.cuda.empty_cache()
+    if legs:
         result["legs"] = legs
 
     # ------------------------------------------------------------------ CPU baselines (oracle port, bounded samples)
@@ -376,7 +386,7 @@ def main() -> int:
             "oracle's per-segment slice-copy loops; same byte accounting as the GPU value",
             "seconds": round(t_cpu, 2),
         }
-        if not args.skip_legs:
+        if "muon" in want:
             u = torch.empty(4096, 4096).normal_(0.0, 1e-3, generator=torch.Generator().manual_seed(MUON_SEED))
             fl, t_ns, ns_reps = 0, 0.0, 0
             while ns_reps < 20 and t_ns < 10.0:

@@ -72,8 +72,9 @@ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_
   *tn = in_group / rows;
 }
 
-template <int BM, int BN, int WM, int WN, int BK, int STAGES>
-__global__ void __launch_bounds__(WM * WN * 64)
+// OCC workgroups are meant to share a CU: the register budget per wave is set for OCC * WM * WN / 4 waves per SIMD.
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int OCC>
+__global__ void __launch_bounds__(WM * WN * 64, (OCC * WM * WN + 3) / 4)
 gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kThreads = WM * WN * 64;
   constexpr int kWaves = WM * WN;
@@ -141,9 +142,10 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // swizzle maps there.  Wave w takes the row groups w, w + kWaves, ...
   const int dl_row = lane / kChunks;
   const int dl_pos = lane % kChunks;
-  auto stream_in = [&](int k0, int stage) {
+  // The P rows and the Q rows of a slab are issued separately: a wave that issues more than four of these loads
+  // back to back stalls on the address queue, and the MFMAs behind them wait with it.
+  auto stream_p = [&](int k0, int stage) {
     __bf16* sp = smem + stage * kStageElems;
-    __bf16* sq = sp + BM * BK;
 #pragma unroll
     for (int i = 0; i < kLoadsP; ++i) {
       const int r0 = (i * kWaves + wave) * kRowsPerLoad;
@@ -151,6 +153,9 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + chunk * 8;
       __builtin_amdgcn_global_load_lds(src, sp + r0 * BK, 16, 0, 0);
     }
+  };
+  auto stream_q = [&](int k0, int stage) {
+    __bf16* sq = smem + stage * kStageElems + BM * BK;
 #pragma unroll
     for (int i = 0; i < kLoadsQ; ++i) {
       const int r0 = (i * kWaves + wave) * kRowsPerLoad;
@@ -204,7 +209,10 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   if (n_slabs > 0) {
 #pragma unroll
     for (int sidx = 0; sidx < STAGES; ++sidx)
-      if (sidx < n_slabs) stream_in(k0_of(sidx), sidx);
+      if (sidx < n_slabs) {
+        stream_p(k0_of(sidx), sidx);
+        stream_q(k0_of(sidx), sidx);
+      }
     if (n_slabs >= STAGES) __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 1) * kLoadsPerSlab) & 0xF) | ((((STAGES - 1) * kLoadsPerSlab) >> 4) << 14));
     else __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
@@ -213,12 +221,18 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   int stage = 0;
   for (int it = 0; it < n_slabs; ++it) {
     const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+    const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
 #pragma unroll
     for (int kk = 0; kk < kSteps; kk += 2) {
       __builtin_amdgcn_s_waitcnt(kWaitLds);
       __builtin_amdgcn_sched_barrier(0);
       load_frags(stage, kk + 1, fa1, fb1);
       __builtin_amdgcn_sched_barrier(0);
+      if (kk == 0 && it >= 1 && it - 1 + STAGES < n_slabs) {
+        // second half of the refill of the stage the previous slab's barrier released (its P rows went out there)
+        stream_q(k0_of(it - 1 + STAGES), prev_stage);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       multiply(fa0, fb0);
       __builtin_amdgcn_sched_barrier(0);
       if (kk + 2 < kSteps) {
@@ -231,7 +245,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
         if (it + STAGES <= n_slabs) __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
         else __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
-        if (it + STAGES < n_slabs) stream_in(k0_of(it + STAGES), stage);
+        if (it + STAGES < n_slabs) stream_p(k0_of(it + STAGES), stage);
         load_frags(next_stage, 0, fa0, fb0);
       } else {
         __builtin_amdgcn_s_waitcnt(kWaitLds);
@@ -391,8 +405,9 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
 
 GemmTuning g_tuning;
 
-template <int BM, int BN, int WM, int WN, int BK, int STAGES>
-int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, hipStream_t stream) {
+template <int BM, int BN, int WM, int WN, int BK, int STAGES, int OCC>
+int launch(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
+  constexpr int blocks_per_cu = OCC;
   Schedule s{};
   s.tiles_m = a.M / BM;
   s.tiles_n = a.N / BN;
@@ -416,9 +431,10 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, int blocks_per_cu, h
   }
   const int blocks = s.full_tiles + (tiles - s.full_tiles) * s.splits;
   constexpr size_t smem_loop = static_cast<size_t>(STAGES) * (BM + BN) * BK * sizeof(uint16_t);
-  constexpr size_t smem_epilogue = static_cast<size_t>(BM > BN ? BM : BN) * ((BM > BN ? BM : BN) + 8) * sizeof(uint16_t);
+  constexpr size_t smem_c = static_cast<size_t>(BM) * (BN + 8) * sizeof(uint16_t), smem_ct = static_cast<size_t>(BN) * (BM + 8) * sizeof(uint16_t);
+  constexpr size_t smem_epilogue = smem_c > smem_ct ? smem_c : smem_ct;
   constexpr size_t smem = smem_loop > smem_epilogue ? smem_loop : smem_epilogue;
-  auto kernel = gemm_nt_kernel<BM, BN, WM, WN, BK, STAGES>;
+  auto kernel = gemm_nt_kernel<BM, BN, WM, WN, BK, STAGES, OCC>;
   static bool configured = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!configured) {
     MFSDP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -456,18 +472,25 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   const int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
   switch (variant) {
     case 2:  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
-      return launch<128, 128, 2, 2, 64, 2>(a, scratch, 2, stream);
+      return launch<128, 128, 2, 2, 64, 2, 2>(a, scratch, stream);
     case 3:  // 256x256 tile, 4 waves of 128x128
-      return launch<256, 256, 2, 2, 64, 2>(a, scratch, 1, stream);
+      return launch<256, 256, 2, 2, 64, 2, 1>(a, scratch, stream);
     case 4:  // 256x256 tile, 8 waves, slabs of 32 four deep
-      return launch<256, 256, 2, 4, 32, 4>(a, scratch, 1, stream);
+      return launch<256, 256, 2, 4, 32, 4, 1>(a, scratch, stream);
     case 5:  // 256x256 tile, 8 waves, slabs of 32 five deep (all 160 KiB of LDS)
-      return launch<256, 256, 2, 4, 32, 5>(a, scratch, 1, stream);
+      return launch<256, 256, 2, 4, 32, 5, 1>(a, scratch, stream);
     case 6:  // 128x128 tile, slabs of 32 four deep, two workgroups per CU
-      return launch<128, 128, 2, 2, 32, 4>(a, scratch, 2, stream);
+      return launch<128, 128, 2, 2, 32, 4, 2>(a, scratch, stream);
+    case 7:  // 256x128 tile, 4 waves of 128x64, slabs of 32 three deep, two workgroups per CU
+      if (a.symmetric) break;
+      return launch<256, 128, 2, 2, 32, 3, 2>(a, scratch, stream);
+    case 8:
+      if (a.symmetric) break;
+      return launch<256, 128, 2, 2, 32, 2, 2>(a, scratch, stream);
     default:  // 256x256 tile, 8 waves of 128x64, slabs of 64 two deep
-      return launch<256, 256, 2, 4, 64, 2>(a, scratch, 1, stream);
+      return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, stream);
   }
+  return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, stream);
 }
 
 }  // namespace mfsdp
