@@ -21,6 +21,7 @@
 #include "mfsdp_common.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace mfsdp {
 namespace {
@@ -129,7 +130,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction: keeps LDS slab addresses scalar
   const int wave_m = wave / WN;
   const int wave_n = wave % WN;
 
@@ -142,27 +143,27 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // swizzle maps there.  Wave w takes the row groups w, w + kWaves, ...
   const int dl_row = lane / kChunks;
   const int dl_pos = lane % kChunks;
-  // The P rows and the Q rows of a slab are issued separately: a wave that issues more than four of these loads
-  // back to back stalls on the address queue, and the MFMAs behind them wait with it.
+  // One load at a time: a wave that issues several of these back to back stalls on the address queue, and its
+  // MFMAs wait with it, so the main loop slips them in between MFMAs.
+  auto load_p = [&](int k0, int stage, int i) {
+    const int r0 = (i * kWaves + wave) * kRowsPerLoad;
+    const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
+    const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + chunk * 8;
+    __builtin_amdgcn_global_load_lds(src, smem + stage * kStageElems + r0 * BK, 16, 0, 0);
+  };
+  auto load_q = [&](int k0, int stage, int i) {
+    const int r0 = (i * kWaves + wave) * kRowsPerLoad;
+    const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
+    const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + chunk * 8;
+    __builtin_amdgcn_global_load_lds(src, smem + stage * kStageElems + BM * BK + r0 * BK, 16, 0, 0);
+  };
   auto stream_p = [&](int k0, int stage) {
-    __bf16* sp = smem + stage * kStageElems;
 #pragma unroll
-    for (int i = 0; i < kLoadsP; ++i) {
-      const int r0 = (i * kWaves + wave) * kRowsPerLoad;
-      const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
-      const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + chunk * 8;
-      __builtin_amdgcn_global_load_lds(src, sp + r0 * BK, 16, 0, 0);
-    }
+    for (int i = 0; i < kLoadsP; ++i) load_p(k0, stage, i);
   };
   auto stream_q = [&](int k0, int stage) {
-    __bf16* sq = smem + stage * kStageElems + BM * BK;
 #pragma unroll
-    for (int i = 0; i < kLoadsQ; ++i) {
-      const int r0 = (i * kWaves + wave) * kRowsPerLoad;
-      const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
-      const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + chunk * 8;
-      __builtin_amdgcn_global_load_lds(src, sq + r0 * BK, 16, 0, 0);
-    }
+    for (int i = 0; i < kLoadsQ; ++i) load_q(k0, stage, i);
   };
 
   f32x16 acc[TM][TN];
@@ -193,7 +194,6 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
   };
-
   // Software pipeline.  STAGES slabs are resident or in flight: the slab being multiplied and the next
   // STAGES - 1, streamed HBM -> LDS while the MFMAs run.  Fragments are double buffered in registers: the
   // TM + TN 128-bit LDS reads of step kk+1 are issued before the MFMAs of step kk (and waited for BEFORE the
@@ -206,18 +206,54 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kInFlight = (STAGES - 2) * kLoadsPerSlab;
   constexpr int kWaitNextSlab = 0x0070 | (kInFlight & 0xF) | ((kInFlight >> 4) << 14);
   bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  // Loads are issued unconditionally, for a slab number clamped to the last one: past the end of the walk they
+  // fetch the last slab once more into a stage nobody reads again.  (A branch around a load in the middle of the
+  // MFMAs makes the register allocator spill the accumulators.)
+  auto k0_clamped = [&](int i) { return k0_of(i < n_slabs ? i : n_slabs - 1); };
   if (n_slabs > 0) {
 #pragma unroll
-    for (int sidx = 0; sidx < STAGES; ++sidx)
-      if (sidx < n_slabs) {
-        stream_p(k0_of(sidx), sidx);
-        stream_q(k0_of(sidx), sidx);
-      }
-    if (n_slabs >= STAGES) __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 1) * kLoadsPerSlab) & 0xF) | ((((STAGES - 1) * kLoadsPerSlab) >> 4) << 14));
-    else __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    for (int sidx = 0; sidx < STAGES; ++sidx) {
+      stream_p(k0_clamped(sidx), sidx);
+      if (sidx + 1 < STAGES) stream_q(k0_clamped(sidx), sidx);  // the Q rows of the last one go out under the first MFMAs
+    }
+    constexpr int kAfterFirst = (STAGES - 2) * kLoadsPerSlab + kLoadsP;
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kAfterFirst & 0xF) | ((kAfterFirst >> 4) << 14));
     __syncthreads();
     load_frags(0, 0, fa0, fb0);
   }
+  // One k16 step: the MFMAs on the fragments in hand (use_a, use_b), the LDS reads of the fragments after them
+  // (stage / kk -> next_a, next_b) and kLoads slab loads, interleaved instruction by instruction: MFMA, LDS read,
+  // MFMA, LDS read, slab load, ...  The matrix pipe is handed to the oldest wave that has an MFMA ready, so
+  // whenever one of the two waves of a SIMD sits at the barrier the other runs alone, and then every clump of
+  // other instructions between two MFMAs is a bubble in the pipe.
+  auto step = [&](const bf16x8 (&use_a)[TM], const bf16x8 (&use_b)[TN], bf16x8 (&next_a)[TM], bf16x8 (&next_b)[TN],
+                  int read_stage, int read_kk, auto loads_tag, auto&& load) {
+    constexpr int kLoads = decltype(loads_tag)::value;
+    constexpr int kMfma = TM * TN, kReads = TM + TN;
+    constexpr int kChunks_ = kLoads > 0 ? kLoads : 1;
+    constexpr int kPer = kMfma / kChunks_;
+    static_assert(kMfma % kChunks_ == 0 && kReads <= kMfma, "step shape");
+    const int off = read_stage * kStageElems + (((read_kk * 2 + frag_half) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
+#pragma unroll
+    for (int c = 0; c < kChunks_; ++c) {
+#pragma unroll
+      for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
+        if (n < TM) next_a[n] = *reinterpret_cast<const bf16x8*>(frag_p + off + n * 32 * BK);
+        else if (n < kReads) next_b[n - TM] = *reinterpret_cast<const bf16x8*>(frag_q + off + (n - TM) * 32 * BK);
+        acc[n / TN][n % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use_a[n / TN], use_b[n % TN], acc[n / TN][n % TN], 0, 0, 0);
+      }
+#pragma unroll
+      for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
+        if (n < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kLoads > 0) {
+        load(c);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
   int stage = 0;
   for (int it = 0; it < n_slabs; ++it) {
     const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
@@ -226,36 +262,30 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int kk = 0; kk < kSteps; kk += 2) {
       __builtin_amdgcn_s_waitcnt(kWaitLds);
       __builtin_amdgcn_sched_barrier(0);
-      load_frags(stage, kk + 1, fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
-      if (kk == 0 && it >= 1 && it - 1 + STAGES < n_slabs) {
+      if (kk == 0) {
         // second half of the refill of the stage the previous slab's barrier released (its P rows went out there)
-        stream_q(k0_of(it - 1 + STAGES), prev_stage);
-        __builtin_amdgcn_sched_barrier(0);
+        const int k0 = k0_clamped(it - 1 + STAGES);
+        step(fa0, fb0, fa1, fb1, stage, kk + 1, std::integral_constant<int, kLoadsQ>{}, [&](int l) { load_q(k0, prev_stage, l); });
+      } else {
+        step(fa0, fb0, fa1, fb1, stage, kk + 1, std::integral_constant<int, 0>{}, [](int) {});
       }
-      multiply(fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
       if (kk + 2 < kSteps) {
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         __builtin_amdgcn_sched_barrier(0);
-        load_frags(stage, kk + 2, fa0, fb0);
-      } else if (it + 1 < n_slabs) {
-        // last step of the slab: the slab after it must have landed; the STAGES - 2 younger ones may be in flight
-        // (near the end of the walk fewer are, then wait for everything)
-        if (it + STAGES <= n_slabs) __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
-        else __builtin_amdgcn_s_waitcnt(0x0070);
-        __syncthreads();
-        if (it + STAGES < n_slabs) stream_p(k0_of(it + STAGES), stage);
-        load_frags(next_stage, 0, fa0, fb0);
+        step(fa1, fb1, fa0, fb0, stage, kk + 2, std::integral_constant<int, 0>{}, [](int) {});
       } else {
-        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        // last step of the slab: the slab after it must have landed (the STAGES - 2 younger ones may be in flight);
+        // behind the barrier this slab's stage is free and its refill starts with the P rows
+        __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        const int k0 = k0_clamped(it + STAGES);
+        step(fa1, fb1, fa0, fb0, next_stage, 0, std::integral_constant<int, kLoadsP>{}, [&](int l) { load_p(k0, stage, l); });
       }
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
     }
     stage = next_stage;
   }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // the loads past the end of the walk have landed too; LDS is free
 
   // ---- K pieces: park the fp32 partial tile (row-major BM x BN); the fix-up kernel sums the pieces and
   // runs the epilogue.  Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
@@ -294,11 +324,19 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kRowChunks = BN / 8, kColChunks = BM / 8;
   __syncthreads();  // every wave is done reading the slab stages
   if (D != nullptr) {
-    for (int c = tid; c < BM * kRowChunks; c += kThreads) {
-      const int r = c / kRowChunks, cc = c - r * kRowChunks;
-      *reinterpret_cast<u32x4*>(stage_c + r * kLdS + cc * 8) =
-          *reinterpret_cast<const u32x4*>(D + static_cast<int64_t>(row0 + r) * a.ldd + col0 + cc * 8);
+    // the D tile streams into LDS (unpadded BM x BN) with all of its loads in flight at once; fetched through
+    // registers, the loads of a thread run one after the other and their latencies add up
+    constexpr int kRowsPerDLoad = 512 / BN;  // D rows one wave-level 1 KiB load covers
+    constexpr int kDLoads = BM / kRowsPerDLoad / kWaves;
+    static_assert(512 % BN == 0 && BM % (kRowsPerDLoad * kWaves) == 0 && kDLoads < 64, "D tile must divide over the waves");
+    const int d_row = lane / kRowChunks, d_chunk = lane % kRowChunks;
+#pragma unroll
+    for (int i = 0; i < kDLoads; ++i) {
+      const int r0 = (i * kWaves + wave) * kRowsPerDLoad;
+      const uint16_t* src = D + static_cast<int64_t>(row0 + r0 + d_row) * a.ldd + col0 + d_chunk * 8;
+      __builtin_amdgcn_global_load_lds(src, stage_c + r0 * BN, 16, 0, 0);
     }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
     __syncthreads();
   }
   const int lcol = wave_n * kWaveN + (lane & 31);
@@ -310,7 +348,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float v = a.alpha * acc[i][j][r];
-        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32]);
+        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * BN + lcol + j * 32]);
         acc[i][j][r] = v;
       }
   if (D != nullptr) __syncthreads();  // the D tile has been consumed
@@ -481,12 +519,6 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
       return launch<256, 256, 2, 4, 32, 5, 1>(a, scratch, stream);
     case 6:  // 128x128 tile, slabs of 32 four deep, two workgroups per CU
       return launch<128, 128, 2, 2, 32, 4, 2>(a, scratch, stream);
-    case 7:  // 256x128 tile, 4 waves of 128x64, slabs of 32 three deep, two workgroups per CU
-      if (a.symmetric) break;
-      return launch<256, 128, 2, 2, 32, 3, 2>(a, scratch, stream);
-    case 8:
-      if (a.symmetric) break;
-      return launch<256, 128, 2, 2, 32, 2, 2>(a, scratch, stream);
     default:  // 256x256 tile, 8 waves of 128x64, slabs of 64 two deep
       return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, stream);
   }
