@@ -232,20 +232,30 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     constexpr int kMfma = TM * TN, kReads = TM + TN;
     constexpr int kChunks_ = kLoads > 0 ? kLoads : 1;
     constexpr int kPer = kMfma / kChunks_;
-    static_assert(kMfma % kChunks_ == 0 && kReads <= kMfma, "step shape");
+    constexpr int kReadsPerMfma = 2;
+    static_assert(kMfma % kChunks_ == 0 && kReads <= kReadsPerMfma * kMfma, "step shape");
     const int off = read_stage * kStageElems + (((read_kk * 2 + frag_half) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
 #pragma unroll
     for (int c = 0; c < kChunks_; ++c) {
 #pragma unroll
       for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
-        if (n < TM) next_a[n] = *reinterpret_cast<const bf16x8*>(frag_p + off + n * 32 * BK);
-        else if (n < kReads) next_b[n - TM] = *reinterpret_cast<const bf16x8*>(frag_q + off + (n - TM) * 32 * BK);
+        // Q fragments first: the MFMAs walk the tile row by row, so the first of them need every Q fragment but
+        // only the first P fragment.  Two reads go out behind each of the first MFMAs, so that the last one has
+        // the rest of the step to come back.
+#pragma unroll
+        for (int r = kReadsPerMfma * n; r < kReadsPerMfma * (n + 1) && r < kReads; ++r) {
+          if (r < TN) next_b[r] = *reinterpret_cast<const bf16x8*>(frag_q + off + r * 32 * BK);
+          else next_a[r - TN] = *reinterpret_cast<const bf16x8*>(frag_p + off + (r - TN) * 32 * BK);
+        }
         acc[n / TN][n % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use_a[n / TN], use_b[n % TN], acc[n / TN][n % TN], 0, 0, 0);
       }
 #pragma unroll
       for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
-        if (n < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        constexpr int kNone = 0;
+        const int reads = kReadsPerMfma * (n + 1) <= kReads ? kReadsPerMfma : (kReadsPerMfma * n < kReads ? kReads - kReadsPerMfma * n : kNone);
+        if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        else if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kLoads > 0) {
