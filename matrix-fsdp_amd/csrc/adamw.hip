@@ -39,34 +39,58 @@ __device__ __forceinline__ void adamw_one(float& p, float g, float& m, float& v,
   p = p + (a.neg_step_size * m) / denom;
 }
 
-template <bool GRAD_BF16>
+template <bool NT, typename T>
+__device__ __forceinline__ T ld(const T* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void st(T* p, T v) {
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
+template <bool GRAD_BF16, int U, bool NT>
 __global__ void __launch_bounds__(256)
 adamw_kernel(float* __restrict__ param, const void* __restrict__ grad, float* __restrict__ exp_avg,
              float* __restrict__ exp_avg_sq, int64_t n_vec, int64_t numel, AdamWArgs a) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_vec; i += stride) {
-    f32x4 p = reinterpret_cast<const f32x4*>(param)[i];
-    f32x4 m = reinterpret_cast<const f32x4*>(exp_avg)[i];
-    f32x4 v = reinterpret_cast<const f32x4*>(exp_avg_sq)[i];
-    f32x4 g;
-    if constexpr (GRAD_BF16) {
-      const u32x2 raw = reinterpret_cast<const u32x2*>(grad)[i];
-      g.x = __uint_as_float(raw.x << 16);
-      g.y = __uint_as_float(raw.x & 0xffff0000u);
-      g.z = __uint_as_float(raw.y << 16);
-      g.w = __uint_as_float(raw.y & 0xffff0000u);
-    } else {
-      g = reinterpret_cast<const f32x4*>(grad)[i];
+  // U vectors per thread and iteration, all of their loads issued before the first use
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * blockDim.x * U + threadIdx.x; base < n_vec; base += stride * U) {
+    f32x4 p[U], m[U], v[U], g[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * 256;
+      if (i < n_vec) {
+        p[u] = ld<NT>(reinterpret_cast<const f32x4*>(param) + i);
+        m[u] = ld<NT>(reinterpret_cast<const f32x4*>(exp_avg) + i);
+        v[u] = ld<NT>(reinterpret_cast<const f32x4*>(exp_avg_sq) + i);
+        if constexpr (GRAD_BF16) {
+          const u32x2 raw = ld<NT>(reinterpret_cast<const u32x2*>(grad) + i);
+          g[u].x = __uint_as_float(raw.x << 16);
+          g[u].y = __uint_as_float(raw.x & 0xffff0000u);
+          g[u].z = __uint_as_float(raw.y << 16);
+          g[u].w = __uint_as_float(raw.y & 0xffff0000u);
+        } else {
+          g[u] = ld<NT>(reinterpret_cast<const f32x4*>(grad) + i);
+        }
+      }
     }
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      float pk = p[k], mk = m[k], vk = v[k];
-      adamw_one(pk, g[k], mk, vk, a);
-      p[k] = pk; m[k] = mk; v[k] = vk;
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * 256;
+      if (i < n_vec) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float pk = p[u][k], mk = m[u][k], vk = v[u][k];
+          adamw_one(pk, g[u][k], mk, vk, a);
+          p[u][k] = pk; m[u][k] = mk; v[u][k] = vk;
+        }
+        st<NT>(reinterpret_cast<f32x4*>(param) + i, p[u]);
+        st<NT>(reinterpret_cast<f32x4*>(exp_avg) + i, m[u]);
+        st<NT>(reinterpret_cast<f32x4*>(exp_avg_sq) + i, v[u]);
+      }
     }
-    reinterpret_cast<f32x4*>(param)[i] = p;
-    reinterpret_cast<f32x4*>(exp_avg)[i] = m;
-    reinterpret_cast<f32x4*>(exp_avg_sq)[i] = v;
   }
   // scalar tail: the elements past the last whole vector (everything when the tensors are not 16-byte aligned)
   for (int64_t i = n_vec * 4 + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += stride) {
@@ -109,14 +133,17 @@ extern "C" int mfsdp_adamw_step(float* param, const void* grad, int grad_dtype, 
   a.bc2_sqrt = static_cast<float>(std::sqrt(bc2));
   a.eps = eps;
   const int64_t n_vec = vec_ok ? numel / 4 : 0;
-  const int64_t work = std::max<int64_t>(n_vec, numel - n_vec * 4);
+  // four vectors per thread with non-temporal accesses (every byte is touched once): 5.7 TB/s against 4.9 TB/s for one
+  // cached vector per thread on 41 M elements
+  constexpr int kVectorsPerThread = 4;
+  const int64_t work = std::max<int64_t>((n_vec + kVectorsPerThread - 1) / kVectorsPerThread, numel - n_vec * 4);
   const int64_t want = std::max<int64_t>(1, (work + 255) / 256);
-  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 8;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 16;
   const dim3 grid(static_cast<uint32_t>(std::min(want, cap)));
   if (grad_dtype == MFSDP_BF16)
-    hipLaunchKernelGGL((adamw_kernel<true>), grid, dim3(256), 0, as_stream(stream), param, grad, exp_avg, exp_avg_sq, n_vec, numel, a);
+    hipLaunchKernelGGL((adamw_kernel<true, kVectorsPerThread, true>), grid, dim3(256), 0, as_stream(stream), param, grad, exp_avg, exp_avg_sq, n_vec, numel, a);
   else
-    hipLaunchKernelGGL((adamw_kernel<false>), grid, dim3(256), 0, as_stream(stream), param, grad, exp_avg, exp_avg_sq, n_vec, numel, a);
+    hipLaunchKernelGGL((adamw_kernel<false, kVectorsPerThread, true>), grid, dim3(256), 0, as_stream(stream), param, grad, exp_avg, exp_avg_sq, n_vec, numel, a);
   MFSDP_CHECK_LAUNCH("adamw_kernel");
   return MFSDP_OK;
 }
