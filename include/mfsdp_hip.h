@@ -186,9 +186,9 @@ int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype
                     void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Kernel selection for experiments (values <= 0 keep the current setting):
- * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves,
- * 2: 128x128 / 4 waves, 3: 256x256 / 4 waves), slabs streamed HBM -> LDS directly (1) or through
- * registers (2), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
+ * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
+ * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU), a reserved argument (slabs always stream
+ * HBM -> LDS directly), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
  * stagger >= 0 sets the K-walk start offset, in 64-element slabs, between consecutive tiles. */
 void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,
                            int max_splits, int stagger);

@@ -34,8 +34,7 @@ struct GemmScratch {
 constexpr int64_t kGemmPartialsBytes = 64ll << 20;
 
 struct GemmTuning {
-  int general_variant = 1;    // 1: 256x256 tile / 8 waves / slabs of 64 two deep, 2: 128x128 / 4 waves, 3: 256x256 / 4 waves,
-                              // 4, 5: as 1 with slabs of 32 four / five deep, 6: as 2 with slabs of 32 four deep
+  int general_variant = 1;    // 1: 256x256 tile / 8 waves / one workgroup per CU, 2: 128x128 tile / 4 waves / two per CU
   int symmetric_variant = 2;
   int direct_to_lds = 1;      // reserved (slabs always stream HBM -> LDS directly)
   int split_remainder = 1;    // split the tiles of the last partial round along K
