@@ -7,6 +7,9 @@ the reference's shard metadata and operator signatures.
 """
 from .core.layout import LayoutSegment, ShardPlan, validate_shard_plan
 from .core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module, managed_params_from_named
+from .api import MixedPrecisionPolicy, fully_shard, matrix_fully_shard
+from .optim.wrapper import MatrixOptimizerConfig, MixedMuonAdamWOptimizer, configure_optimizer
+from .runtime.param_group import FSDPLifecycleState, MatrixFSDPParamGroup
 
 __all__ = [
     "LayoutSegment",
@@ -16,4 +19,12 @@ __all__ = [
     "ParamShardHint",
     "managed_params_from_module",
     "managed_params_from_named",
+    "MixedPrecisionPolicy",
+    "fully_shard",
+    "matrix_fully_shard",
+    "MatrixOptimizerConfig",
+    "MixedMuonAdamWOptimizer",
+    "configure_optimizer",
+    "FSDPLifecycleState",
+    "MatrixFSDPParamGroup",
 ]

@@ -1,0 +1,111 @@
+"""``fully_shard`` / ``matrix_fully_shard``: wrap a module's parameters into one flat-buffer unit.
+
+The entry points keep the reference's names and the arguments that matter on a
+single device (matrix_fsdp/api.py:213-263 ``fully_shard``, :266-330
+``matrix_fully_shard``).  There is no process group here: ``world_size`` and
+``rank`` say which simulated world the unit is sharded for (default: a world
+of one, the reference's single-rank path).  Arguments that only steer
+collectives, prefetching, offload or the planner families are not accepted.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Mapping
+
+import torch
+from torch import nn
+
+from .core.layout import ShardPlan
+from .core.managed_param import ManagedParam, ParamShardHint
+from .runtime.param_group import MatrixFSDPParamGroup
+
+
+@dataclass(frozen=True)
+class MixedPrecisionPolicy:
+    """Field-compatible with ``torch.distributed.fsdp.MixedPrecisionPolicy``, which is accepted as well."""
+
+    param_dtype: torch.dtype | None = None
+    reduce_dtype: torch.dtype | None = None
+    output_dtype: torch.dtype | None = None
+    cast_forward_inputs: bool = True
+
+
+_DEFAULT_MP_POLICY = MixedPrecisionPolicy()
+
+
+def validate_mixed_precision_policy(mp_policy) -> None:
+    for name in ("param_dtype", "reduce_dtype", "output_dtype"):
+        dtype = getattr(mp_policy, name, None)
+        if dtype is not None and not (isinstance(dtype, torch.dtype) and dtype.is_floating_point):
+            raise ValueError(f"mp_policy.{name} must be a floating-point torch.dtype or None, got {dtype!r}.")
+
+
+def matrix_fully_shard(
+    module: nn.Module,
+    *,
+    world_size: int = 1,
+    rank: int = 0,
+    planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
+    shard_hints: Mapping[str, ParamShardHint] | None = None,
+    ignored_params: set[nn.Parameter] | None = None,
+    reshard_after_forward: bool = True,
+    mp_policy=_DEFAULT_MP_POLICY,
+) -> nn.Module:
+    """Turns ``module`` into one unit: its parameters (those no nested unit
+    manages yet) move into a flat buffer sharded by ``planner`` for the
+    simulated world, become views of rank ``rank``'s local shard, and forward /
+    backward hooks unshard and reshard them.  Returns ``module``."""
+    validate_mixed_precision_policy(mp_policy)
+    if getattr(module, "_matrix_fsdp_param_group", None) is not None:
+        raise ValueError("module is already wrapped by matrix_fully_shard().")
+    MatrixFSDPParamGroup(
+        module,
+        world_size=world_size,
+        rank=rank,
+        planner=planner,
+        shard_hints=shard_hints,
+        ignored_params=ignored_params,
+        reshard_after_forward=reshard_after_forward,
+        param_dtype=getattr(mp_policy, "param_dtype", None),
+        reduce_dtype=getattr(mp_policy, "reduce_dtype", None),
+        output_dtype=getattr(mp_policy, "output_dtype", None),
+        cast_forward_inputs=getattr(mp_policy, "cast_forward_inputs", True),
+    )
+    return module
+
+
+def fully_shard(
+    module: nn.Module,
+    *,
+    world_size: int = 1,
+    rank: int = 0,
+    reshard_after_forward: bool | None = None,
+    shard_placement_fn: Callable[[nn.Parameter], ParamShardHint | None] | None = None,
+    mp_policy=_DEFAULT_MP_POLICY,
+    ignored_params: set[nn.Parameter] | None = None,
+    planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
+) -> nn.Module:
+    """FSDP2-style spelling (matrix_fsdp/api.py:213-263): ``shard_placement_fn``
+    maps a parameter to a ``ParamShardHint`` (or ``None``); ``reshard_after_forward``
+    defaults to ``True``."""
+    hints: dict[str, ParamShardHint] = {}
+    if shard_placement_fn is not None:
+        ignored = {id(p) for p in ignored_params or ()}
+        for fqn, param in module.named_parameters():
+            if id(param) in ignored or getattr(param, "_matrix_fsdp_managed", False):
+                continue
+            hint = shard_placement_fn(param)
+            if hint is not None:
+                if not isinstance(hint, ParamShardHint):
+                    raise TypeError(f"shard_placement_fn must return ParamShardHint or None, got {type(hint).__name__} for {fqn}.")
+                hints[fqn] = hint
+    return matrix_fully_shard(
+        module,
+        world_size=world_size,
+        rank=rank,
+        planner=planner,
+        shard_hints=hints or None,
+        ignored_params=ignored_params,
+        reshard_after_forward=True if reshard_after_forward is None else bool(reshard_after_forward),
+        mp_policy=mp_policy,
+    )

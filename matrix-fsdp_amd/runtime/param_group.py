@@ -1,0 +1,265 @@
+"""``MatrixFSDPParamGroup``: the forward / backward lifecycle of one unit on a single HIP device.
+
+A unit is a module whose parameters share one ``MatrixFlatBuffer``.  Between
+steps the parameters are views of the rank's local shard (what the optimizer
+updates); around the unit's forward and backward they are views of the full
+buffer.  The hooks below drive that swap the way the reference's unit does
+(matrix_fsdp/runtime/fsdp_unit.py:250-310 registration, :1024-1192 forward
+hooks, :1384-1421 post-accumulate-grad counting, :1470-1560 backward
+finalisation), with everything that needs more than one process left out:
+no process group (a world of size ``W`` is simulated in memory by the flat
+buffer), no prefetch scheduler, no communication streams, no offload.
+
+States (matrix_fsdp/runtime/fsdp_unit.py:63-66):
+``SHARDED`` -> pre-forward -> ``UNSHARDED`` -> post-forward ->
+``FORWARD_RESHARDED`` (only with ``reshard_after_forward``) -> pre-backward ->
+``UNSHARDED`` -> last gradient accumulated -> ``SHARDED`` with ``param.grad``
+pointing into the reduced local gradient shard.
+"""
+from __future__ import annotations
+
+from enum import Enum
+from typing import Callable, Iterable, Mapping
+
+import torch
+from torch import nn
+from torch.autograd import Variable
+
+from ..core.layout import ShardPlan
+from ..core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module
+from ..core.plans import contiguous_even_plan, fsdp2_chunk_plan
+from .flat_buffer import MatrixFlatBuffer
+
+Planner = Callable[[list[ManagedParam], int], ShardPlan]
+
+_MANAGED_ATTR = "_matrix_fsdp_managed"
+
+
+class FSDPLifecycleState(str, Enum):
+    SHARDED = "sharded"
+    UNSHARDED = "unsharded"
+    FORWARD_RESHARDED = "forward_resharded"
+
+
+def default_planner(managed_params: list[ManagedParam], world_size: int) -> ShardPlan:
+    """Per-parameter even chunks when every parameter divides by the world
+    size (matrix_fsdp/planning/planner.py:428-487), otherwise the rank-contiguous
+    even split of the flat buffer (planner.py:46-56)."""
+    if all(mp.numel % world_size == 0 for mp in managed_params):
+        return fsdp2_chunk_plan(managed_params, world_size)
+    return contiguous_even_plan(managed_params[-1].end, world_size)
+
+
+def _floating_tensors_to(obj, dtype: torch.dtype):
+    """Floating-point tensors anywhere in ``obj`` cast to ``dtype``
+    (the reference's ``cast_floating_tensors``)."""
+    if isinstance(obj, torch.Tensor):
+        return obj.to(dtype) if obj.is_floating_point() and obj.dtype != dtype else obj
+    if isinstance(obj, (list, tuple)):
+        return type(obj)(_floating_tensors_to(o, dtype) for o in obj)
+    if isinstance(obj, dict):
+        return {k: _floating_tensors_to(v, dtype) for k, v in obj.items()}
+    return obj
+
+
+def _tensors_requiring_grad(obj) -> Iterable[torch.Tensor]:
+    if isinstance(obj, torch.Tensor):
+        if obj.requires_grad:
+            yield obj
+    elif isinstance(obj, (list, tuple)):
+        for o in obj:
+            yield from _tensors_requiring_grad(o)
+    elif isinstance(obj, dict):
+        for o in obj.values():
+            yield from _tensors_requiring_grad(o)
+
+
+class MatrixFSDPParamGroup:
+    def __init__(
+        self,
+        module: nn.Module,
+        *,
+        world_size: int = 1,
+        rank: int = 0,
+        planner: Planner | None = None,
+        shard_hints: Mapping[str, ParamShardHint] | None = None,
+        ignored_params: set[nn.Parameter] | None = None,
+        reshard_after_forward: bool = True,
+        param_dtype: torch.dtype | None = None,
+        reduce_dtype: torch.dtype | None = None,
+        output_dtype: torch.dtype | None = None,
+        cast_forward_inputs: bool = True,
+    ) -> None:
+        if world_size < 1 or not 0 <= rank < world_size:
+            raise ValueError(f"rank {rank} is outside a world of {world_size}.")
+        self.module = module
+        self.world_size = world_size
+        self.rank = rank
+        self.planner = planner or default_planner
+        self.shard_hints = shard_hints
+        self.ignored_params = set(ignored_params or ())
+        self.reshard_after_forward_enabled = bool(reshard_after_forward)
+        self.param_dtype = param_dtype
+        self.reduce_dtype = reduce_dtype
+        self.output_dtype = output_dtype
+        self.cast_forward_inputs = cast_forward_inputs
+        self.managed_params: list[ManagedParam] = []
+        self.flat_buffer: MatrixFlatBuffer | None = None
+        self.shard_plan: ShardPlan | None = None
+        self.lifecycle_state = FSDPLifecycleState.SHARDED
+        self.events: list[str] = []
+        self._handles: list = []
+        self._seen_param_ids: set[int] = set()
+        self._expected_param_ids: set[int] = set()
+        self._backward_callback_queued = False
+        self._finalized_after_backward = True
+        self.init()
+
+    # ------------------------------------------------------------------ set-up
+    def init(self) -> None:
+        # parameters a nested unit already manages stay with that unit
+        taken = {p for p in self.module.parameters() if getattr(p, _MANAGED_ATTR, False)}
+        self.managed_params = list(
+            managed_params_from_module(self.module, shard_hints=self.shard_hints, ignored_params=self.ignored_params | taken)
+        )
+        self.module._matrix_fsdp_param_group = self  # type: ignore[attr-defined]
+        if not self.managed_params:
+            return
+        plan = self.planner(self.managed_params, self.world_size)
+        if len(plan.shard_sizes) != self.world_size:
+            raise ValueError(f"planner returned a plan for {len(plan.shard_sizes)} ranks, expected {self.world_size}.")
+        self.shard_plan = plan
+        self.flat_buffer = MatrixFlatBuffer(
+            self.managed_params, plan, self.rank, param_dtype=self.param_dtype, reduce_dtype=self.reduce_dtype
+        )
+        buffers = list(getattr(self.module, "_matrix_fsdp_flat_buffers", ()))
+        self.module._matrix_fsdp_flat_buffers = (*buffers, self.flat_buffer)  # type: ignore[attr-defined]
+        for mp in self.managed_params:
+            setattr(mp.param, _MANAGED_ATTR, True)
+            self._expected_param_ids.add(id(mp.param))
+            self._handles.append(mp.param.register_post_accumulate_grad_hook(self._post_accumulate_grad))
+        self._handles.append(self.module.register_forward_pre_hook(self._pre_forward, with_kwargs=True))
+        self._handles.append(self.module.register_forward_hook(self._post_forward, with_kwargs=True))
+        self._record("init")
+
+    def _record(self, event: str) -> None:
+        self.events.append(event)
+        if len(self.events) > 256:
+            del self.events[:128]
+
+    def remove_hooks(self) -> None:
+        for handle in self._handles:
+            handle.remove()
+        self._handles.clear()
+
+    # ------------------------------------------------------------------ shard / unshard
+    def _single_rank_alias(self) -> bool:
+        """A world of one with no compute-dtype cast: the local shard *is* the
+        full buffer (matrix_fsdp/runtime/flat_buffer.py:320-327)."""
+        fb = self.flat_buffer
+        return self.world_size == 1 and fb.layout.packed_rank_shards_are_full_tensor_order and fb._param_compute_dtype() == fb.local_shard.dtype
+
+    def unshard(self, reason: str = "manual") -> None:
+        if self.flat_buffer is None or self.lifecycle_state == FSDPLifecycleState.UNSHARDED:
+            return
+        fb = self.flat_buffer
+        if self._single_rank_alias():
+            fb.full_buffer = fb.local_shard
+            fb.use_full_param_buffer()
+        else:
+            fb.unshard()
+        self.lifecycle_state = FSDPLifecycleState.UNSHARDED
+        self._record(f"unshard:{reason}")
+
+    def reshard(self, reason: str = "manual") -> None:
+        if self.flat_buffer is None:
+            return
+        self.flat_buffer.use_local_shards()
+        self.lifecycle_state = FSDPLifecycleState.SHARDED
+        self._record(f"reshard:{reason}")
+
+    # ------------------------------------------------------------------ forward hooks
+    def _pre_forward(self, module, args, kwargs):
+        if self.flat_buffer is None:
+            return args, kwargs
+        if not self._finalized_after_backward and self.lifecycle_state == FSDPLifecycleState.FORWARD_RESHARDED:
+            raise RuntimeError(
+                "reshard_after_forward=True does not support running another forward before the previous forward has entered backward."
+            )
+        self._seen_param_ids.clear()
+        self._record("pre_forward")
+        self.unshard("pre_forward")
+        if self.cast_forward_inputs and self.param_dtype is not None:
+            args = _floating_tensors_to(args, self.param_dtype)
+            kwargs = _floating_tensors_to(kwargs, self.param_dtype)
+        return args, kwargs
+
+    def _post_forward(self, module, args, kwargs, output):
+        if self.flat_buffer is None:
+            return output
+        grad_enabled = torch.is_grad_enabled()
+        outputs_with_grad = list(_tensors_requiring_grad(output)) if grad_enabled else []
+        if outputs_with_grad:
+            self._finalized_after_backward = False
+            for tensor in outputs_with_grad:
+                tensor.register_hook(self._pre_backward)
+        if self.reshard_after_forward_enabled or not outputs_with_grad:
+            self.flat_buffer.use_local_shards()
+            self.lifecycle_state = FSDPLifecycleState.FORWARD_RESHARDED if outputs_with_grad else FSDPLifecycleState.SHARDED
+            self._record("reshard:post_forward")
+        if self.output_dtype is not None:
+            output = _floating_tensors_to(output, self.output_dtype)
+        return output
+
+    # ------------------------------------------------------------------ backward
+    def _pre_backward(self, grad: torch.Tensor) -> torch.Tensor:
+        if not self._backward_callback_queued:
+            self._backward_callback_queued = True
+            Variable._execution_engine.queue_callback(self._post_backward_callback)
+        if self.lifecycle_state != FSDPLifecycleState.UNSHARDED and not self._finalized_after_backward:
+            self._record("pre_backward")
+            self.unshard("pre_backward")
+        return grad
+
+    def _post_accumulate_grad(self, param: torch.Tensor) -> None:
+        if id(param) not in self._expected_param_ids:
+            return
+        self._seen_param_ids.add(id(param))
+        if len(self._seen_param_ids) == len(self._expected_param_ids) and self.lifecycle_state == FSDPLifecycleState.UNSHARDED:
+            self.finalize_backward()
+
+    def _post_backward_callback(self) -> None:
+        """End of the autograd pass: units whose parameters did not all receive
+        a gradient are finalised here."""
+        self._backward_callback_queued = False
+        if not self._finalized_after_backward:
+            self.finalize_backward()
+
+    def finalize_backward(self) -> None:
+        """Per-parameter grads -> reduce-scatter input -> this rank's reduced
+        gradient shard; parameters and their grads become local-shard views
+        again."""
+        fb = self.flat_buffer
+        if fb is None or self._finalized_after_backward:
+            return
+        bucket = fb.collect_grad_bucket()
+        if bucket.param_grads:
+            missing = [mp for mp in self.managed_params if all(pg.managed_param is not mp for pg in bucket.param_grads)]
+            if missing:
+                # parameters without a gradient contribute zeros, as a reduce-scatter of an untouched workspace would
+                zeros = [(mp, torch.zeros(mp.numel, dtype=bucket.param_grads[0].grad.dtype, device=fb.device)) for mp in missing]
+                from .grad_bucket import BucketParamGrad, MatrixGradBucket
+
+                by_fqn = {pg.managed_param.fqn: pg for pg in bucket.param_grads}
+                by_fqn.update({mp.fqn: BucketParamGrad(mp, z) for mp, z in zeros})
+                ordered = tuple(by_fqn[mp.fqn] for mp in self.managed_params)
+                bucket = MatrixGradBucket(ordered, bucket.total_numel, bucket.shard_sizes, bucket.rank_segments)
+            fb.reduce_grad_bucket_to_local_shard(bucket)
+            fb.use_local_shards()
+            fb.use_local_grad_shard()
+        else:
+            fb.use_local_shards()
+        self.lifecycle_state = FSDPLifecycleState.SHARDED
+        self._finalized_after_backward = True
+        self._seen_param_ids.clear()
+        self._record("finalize_backward")

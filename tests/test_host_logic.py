@@ -201,3 +201,27 @@ def test_grad_fill_runs_match_the_oracle_on_random_layouts():
         want = torch.full((world * max_shard,), -1.0)
         O.fill_reduce_scatter_input(params, grads, plan.shard_sizes, plan.rank_segments, total, want)
         assert torch.equal(have, want)
+
+
+def test_fully_shard_host_rules():
+    """What the lifecycle shell decides on the host: the default plan, parameter ownership of nested units, and
+    that nothing runs without a HIP device (there is no CPU fallback)."""
+    from matrix_fsdp_amd import MixedPrecisionPolicy, fully_shard
+    from matrix_fsdp_amd.api import validate_mixed_precision_policy
+    from matrix_fsdp_amd.core.managed_param import managed_params_from_module
+    from matrix_fsdp_amd.runtime.param_group import default_planner
+
+    module = torch.nn.Sequential(torch.nn.Linear(8, 4), torch.nn.Linear(4, 3))
+    mps = list(managed_params_from_module(module))
+    chunked = default_planner(mps, 1)
+    assert chunked.shard_sizes == (sum(mp.numel for mp in mps),)
+    ragged = default_planner(mps, 4)  # 3 x 4 weights and a bias of 3 do not divide by 4: rank-contiguous even split
+    assert sum(ragged.shard_sizes) == mps[-1].end and max(ragged.shard_sizes) - min(ragged.shard_sizes) <= 1
+    even = default_planner(mps[:2], 4)
+    assert even.shard_sizes == (9, 9, 9, 9) and len(even.rank_segments[0]) == 2  # a chunk of every parameter
+    with pytest.raises(RuntimeError, match="HIP device"):
+        fully_shard(module)
+    with pytest.raises(ValueError, match="floating-point"):
+        validate_mixed_precision_policy(MixedPrecisionPolicy(reduce_dtype=torch.int64))
+    with pytest.raises(TypeError, match="ParamShardHint"):
+        fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: "muon")
