@@ -17,7 +17,13 @@ from torch import nn
 
 from .core.layout import ShardPlan
 from .core.managed_param import ManagedParam, ParamShardHint
+from .planning.owner_plans import MuonOwnerPlanner
+from .planning.shard_hint import build_shard_hints
 from .runtime.param_group import MatrixFSDPParamGroup
+
+# optimizer_policy values of fully_shard (matrix_fsdp/api.py:43-54)
+_MUON_OPTIMIZER_POLICIES = {"mixed_muon_adamw", "muon_adamw", "muon_shard_aware", "muon"}
+_NOOP_OPTIMIZER_POLICIES = {"default", "none", "adamw", "sgd"}
 
 
 @dataclass(frozen=True)
@@ -84,11 +90,28 @@ def fully_shard(
     mp_policy=_DEFAULT_MP_POLICY,
     ignored_params: set[nn.Parameter] | None = None,
     planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
+    optimizer_policy: str | None = None,
 ) -> nn.Module:
     """FSDP2-style spelling (matrix_fsdp/api.py:213-263): ``shard_placement_fn``
     maps a parameter to a ``ParamShardHint`` (or ``None``); ``reshard_after_forward``
-    defaults to ``True``."""
+    defaults to ``True``.  A Muon ``optimizer_policy`` (``"muon"``,
+    ``"mixed_muon_adamw"``, ...) derives the hints from the module structure
+    (``build_shard_hints``) and keeps every parameter whole on an owner rank
+    (``MuonOwnerPlanner``; pass one planner object to all units to balance the
+    ranks across units)."""
     hints: dict[str, ParamShardHint] = {}
+    if optimizer_policy is not None:
+        policy = optimizer_policy.lower()
+        if policy in _MUON_OPTIMIZER_POLICIES:
+            if shard_placement_fn is not None:
+                raise ValueError("fully_shard optimizer_policy cannot be combined with shard_placement_fn.")
+            skip = {id(p) for p in ignored_params or ()}
+            mine = {fqn for fqn, p in module.named_parameters() if id(p) not in skip and not getattr(p, "_matrix_fsdp_managed", False)}
+            hints = {fqn: hint for fqn, hint in build_shard_hints(module).items() if fqn in mine}
+            planner = planner or MuonOwnerPlanner()
+        elif policy not in _NOOP_OPTIMIZER_POLICIES:
+            allowed = sorted(_MUON_OPTIMIZER_POLICIES | _NOOP_OPTIMIZER_POLICIES)
+            raise ValueError(f"Unknown fully_shard optimizer_policy={optimizer_policy!r}; expected one of {allowed}.")
     if shard_placement_fn is not None:
         ignored = {id(p) for p in ignored_params or ()}
         for fqn, param in module.named_parameters():

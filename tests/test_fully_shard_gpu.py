@@ -249,3 +249,53 @@ def test_lifecycle_rules():
         fully_shard(model)
     with pytest.raises(ValueError, match="floating-point"):
         fully_shard(nn.Linear(4, 4).to(DEV), mp_policy=MixedPrecisionPolicy(param_dtype=torch.int32))
+
+
+def test_muon_optimizer_policy_in_a_simulated_world_of_two():
+    """``optimizer_policy="muon"``: hints from the module structure, whole-parameter owners balanced over the
+    units by one shared planner, Muon on the matrices rank 0 owns and AdamW on its vectors.  The twin trains
+    everything and puts back what rank 0 does not own."""
+    from matrix_fsdp_amd.planning import MuonOwnerPlanner, owner_ranks
+
+    world, rank = 2, 0
+    model, twin = make_pair(seed=10)
+    planner = MuonOwnerPlanner()
+    for unit in [*model.blocks, model]:
+        fully_shard(unit, world_size=world, rank=rank, optimizer_policy="muon", planner=planner, reshard_after_forward=False)
+    owned = {}
+    for prefix, unit in [("blocks.0.", model.blocks[0]), ("blocks.1.", model.blocks[1]), ("", model)]:
+        group = unit._matrix_fsdp_param_group
+        for mp in group.managed_params:
+            ranks = owner_ranks(group.shard_plan, mp)
+            assert len(ranks) == 1  # never cut
+            owned[prefix + mp.fqn] = ranks[0] == rank
+    assert 0 < sum(owned.values()) < len(owned)
+    assert abs(planner.rank_units[0] - planner.rank_units[1]) <= max(p.numel() for p in twin.parameters())
+    opt = configure_optimizer(model, "mixed_muon_adamw", lr=1e-3, weight_decay=0.0)
+    assert all(p.ndim == 2 for p in opt.muon_params) and len(opt.muon_params) == sum(owned[n] and p.ndim == 2 for n, p in twin.named_parameters())
+    twin_named = dict(twin.named_parameters())
+    defaults = opt.defaults
+    ref_muon = torch.optim.Muon([p for n, p in twin_named.items() if p.ndim == 2], **{k: defaults["muon"][k] for k in ("lr", "weight_decay", "momentum", "nesterov", "ns_coefficients", "eps", "ns_steps", "adjust_lr_fn")})
+    ref_adamw = torch.optim.AdamW([p for n, p in twin_named.items() if p.ndim != 2], **{k: defaults["adamw"][k] for k in ("lr", "betas", "eps", "weight_decay")}, foreach=False)
+    start = named_full_params(twin)
+    for x, y in batches(2, seed=11):
+        torch.nn.functional.mse_loss(model(x), y).backward()
+        opt.step()
+        opt.zero_grad()
+        before = {n: p.detach().clone() for n, p in twin_named.items()}
+        torch.nn.functional.mse_loss(twin(x), y).backward()
+        ref_muon.step()
+        ref_adamw.step()
+        ref_muon.zero_grad()
+        ref_adamw.zero_grad()
+        with torch.no_grad():
+            for n, p in twin_named.items():
+                if not owned[n]:
+                    p.copy_(before[n])
+    for n, p in model.named_parameters():
+        if owned[n]:
+            want = twin_named[n].detach().float().cpu()
+            tol = 2e-2 if want.ndim == 2 else 2e-3
+            assert rel(p.detach().float().cpu() - start[n], want - start[n]) < tol, n
+        else:
+            assert p.numel() == 0, n
