@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--skip-mixed", action="store_true", help="skip the hidden5120 mixed-step leg")
     ap.add_argument("--legs", default="rows,muon,adamw,mixed", help="comma list of the extra legs to run: rows (hidden2048 row split), muon, adamw, mixed")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
-    ap.add_argument("--no-launch-events", action="store_true", help="no per-launch HIP events inside the timed region")
+    ap.add_argument("--no-launch-events", action="store_true", help="no HIP events inside the timed region (launch time from the wall clock)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain Tensor.copy_ of 1 GiB (a copy kernel of known size, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -119,24 +119,18 @@ def main() -> int:
     launch_events = []
 
     def step(record: bool) -> None:
+        # one pair of HIP events around the step's 2 * layers launches (on the stream they are launched on): events
+        # around every single launch cost about 5 % of the throughput they are meant to measure
+        if record:
+            a, b = event_pair(torch)
+            a.record()
         for i in range(layers):
-            if record:
-                a, b = event_pair(torch)
-                a.record()
-                pack.run((fulls[i],), gathered[i])
-                b.record()
-                launch_events.append((a, b))
-            else:
-                pack.run((fulls[i],), gathered[i])
+            pack.run((fulls[i],), gathered[i])
         for i in range(layers):
-            if record:
-                a, b = event_pair(torch)
-                a.record()
-                unpack.run((gathered[i],), outs[i])
-                b.record()
-                launch_events.append((a, b))
-            else:
-                unpack.run((gathered[i],), outs[i])
+            unpack.run((gathered[i],), outs[i])
+        if record:
+            b.record()
+            launch_events.append((a, b))
 
     if args.calibrate_copy:
         cal_src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
@@ -161,7 +155,7 @@ def main() -> int:
         print("unpack(pack(x)) != x", file=sys.stderr)
         return 1
     if launch_events:
-        avg_launch_ms = sum(a.elapsed_time(b) for a, b in launch_events) / len(launch_events)
+        avg_launch_ms = sum(a.elapsed_time(b) for a, b in launch_events) / (len(launch_events) * 2 * layers)
     else:
         avg_launch_ms = ms_per_step / (2 * layers)
     achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9
@@ -177,7 +171,7 @@ def main() -> int:
         "traffic": 812_800_000 if layers > 0 else None,
         "algorithmic_bytes_per_launch": bytes_per_launch,
         "avg_launch_ms": round(avg_launch_ms, 5),
-        "launches_timed": len(launch_events),
+        "launches_timed": len(launch_events) * 2 * layers,
     }
     result = {
         "metric": "pack/unpack GB/s (% HBM peak); Muon NS TFLOP/s + ms/step at hidden4096",
