@@ -302,58 +302,57 @@ def main() -> int:
         # -------------------------------------------------------------- hidden5120 mixed step, rank 0 of a simulated world of 4:
         # pack + unpack of the 40 rank-major owner-layout layer buffers (uneven shards, padded staging), AdamW on the fp32
         # tail shard, Muon on the 50 matrices this rank owns
-        if True:
-            w5 = HIDDEN5120
-            progs = {}
-            for k in range(w5.world_size):  # the owner pattern repeats every world_size layers
-                plan5 = w5.owner_layout(k)[2]
-                progs[k] = (plan5, pack_program(plan5, torch.bfloat16, device=dev), unpack_program(plan5, torch.bfloat16, device=dev))
-            gen5 = torch.Generator(device=dev).manual_seed(w5.seed)
-            full5 = [torch.empty(w5.total_numel, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02, generator=gen5) for _ in range(w5.layers)]
-            gath5 = [torch.empty(w5.world_size * progs[i % w5.world_size][0].max_shard_size, dtype=torch.bfloat16, device=dev) for i in range(w5.layers)]
-            out5 = [torch.empty(w5.total_numel, dtype=torch.bfloat16, device=dev) for _ in range(w5.layers)]
+        w5 = HIDDEN5120
+        progs = {}
+        for k in range(w5.world_size):  # the owner pattern repeats every world_size layers
+            plan5 = w5.owner_layout(k)[2]
+            progs[k] = (plan5, pack_program(plan5, torch.bfloat16, device=dev), unpack_program(plan5, torch.bfloat16, device=dev))
+        gen5 = torch.Generator(device=dev).manual_seed(w5.seed)
+        full5 = [torch.empty(w5.total_numel, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02, generator=gen5) for _ in range(w5.layers)]
+        gath5 = [torch.empty(w5.world_size * progs[i % w5.world_size][0].max_shard_size, dtype=torch.bfloat16, device=dev) for i in range(w5.layers)]
+        out5 = [torch.empty(w5.total_numel, dtype=torch.bfloat16, device=dev) for _ in range(w5.layers)]
 
-            def copies5():
-                for i in range(w5.layers):
-                    progs[i % w5.world_size][1].run((full5[i],), gath5[i])
-                for i in range(w5.layers):
-                    progs[i % w5.world_size][2].run((gath5[i],), out5[i])
+        def copies5():
+            for i in range(w5.layers):
+                progs[i % w5.world_size][1].run((full5[i],), gath5[i])
+            for i in range(w5.layers):
+                progs[i % w5.world_size][2].run((gath5[i],), out5[i])
 
-            t_copy, _ = time_launches(torch, copies5, 5, 2)
-            assert torch.equal(out5[1], full5[1])
-            copy_bytes = sum(progs[i % w5.world_size][1].bytes_moved + progs[i % w5.world_size][2].bytes_moved for i in range(w5.layers))
-            del full5, gath5, out5, progs
-            torch.cuda.empty_cache()
+        t_copy, _ = time_launches(torch, copies5, 5, 2)
+        assert torch.equal(out5[1], full5[1])
+        copy_bytes = sum(progs[i % w5.world_size][1].bytes_moved + progs[i % w5.world_size][2].bytes_moved for i in range(w5.layers))
+        del full5, gath5, out5, progs
+        torch.cuda.empty_cache()
 
-            owned = [s.shape for layer in range(w5.layers) for s, o in zip(w5.specs, w5.owner_ranks(layer)) if o == 0 and len(s.shape) == 2]
-            mats5 = []
-            for shape in owned:
-                p = torch.empty(shape, device=dev).normal_(0.0, 0.02, generator=gen5)
-                g = torch.empty(shape, device=dev).normal_(0.0, 1e-3, generator=gen5).bfloat16().float()
-                mats5.append((p, g, torch.zeros(shape, device=dev)))
-            pa = torch.empty(n_adam, device=dev).normal_(0.0, 0.02, generator=gen5)
-            ga = torch.empty(n_adam, device=dev).normal_(0.0, 1e-3, generator=gen5)
-            ma, va = torch.zeros(n_adam, device=dev), torch.zeros(n_adam, device=dev)
+        owned = [s.shape for layer in range(w5.layers) for s, o in zip(w5.specs, w5.owner_ranks(layer)) if o == 0 and len(s.shape) == 2]
+        mats5 = []
+        for shape in owned:
+            p = torch.empty(shape, device=dev).normal_(0.0, 0.02, generator=gen5)
+            g = torch.empty(shape, device=dev).normal_(0.0, 1e-3, generator=gen5).bfloat16().float()
+            mats5.append((p, g, torch.zeros(shape, device=dev)))
+        pa = torch.empty(n_adam, device=dev).normal_(0.0, 0.02, generator=gen5)
+        ga = torch.empty(n_adam, device=dev).normal_(0.0, 1e-3, generator=gen5)
+        ma, va = torch.zeros(n_adam, device=dev), torch.zeros(n_adam, device=dev)
 
-            def update5():
-                F.adamw_step(pa, ga, ma, va, 1, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
-                for p, g, buf in mats5:
-                    F.muon_step(p, g, buf, workspace=ws, **kw)
+        def update5():
+            F.adamw_step(pa, ga, ma, va, 1, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+            for p, g, buf in mats5:
+                F.muon_step(p, g, buf, workspace=ws, **kw)
 
-            t_upd, _ = time_launches(torch, update5, 3, 1)
-            flops5 = sum(5 * (4 * min(sh) ** 2 * max(sh) + 2 * min(sh) ** 3) for sh in owned)
-            legs["hidden5120_mixed_step_rank0_of_4"] = {
-                "ms_per_step": round(t_copy + t_upd, 3),
-                "copies_ms": round(t_copy, 4),
-                "copies_GBps": round(copy_bytes / (t_copy * 1e-3) / 1e9, 1),
-                "update_ms": round(t_upd, 3),
-                "muon_matrices": len(owned),
-                "ns_TFLOPs_reference_flop_count": round(flops5 / (t_upd * 1e-3) / 1e12, 1),
-                "note": "40 owner-layout layer buffers packed and unpacked (padded staging of uneven shards, zero-filled pad "
-                "tails counted as written bytes), AdamW on the 41M-element fp32 tail shard, Muon on every 4th matrix",
-            }
-            del mats5, pa, ga, ma, va
-            torch.cuda.empty_cache()
+        t_upd, _ = time_launches(torch, update5, 3, 1)
+        flops5 = sum(5 * (4 * min(sh) ** 2 * max(sh) + 2 * min(sh) ** 3) for sh in owned)
+        legs["hidden5120_mixed_step_rank0_of_4"] = {
+            "ms_per_step": round(t_copy + t_upd, 3),
+            "copies_ms": round(t_copy, 4),
+            "copies_GBps": round(copy_bytes / (t_copy * 1e-3) / 1e9, 1),
+            "update_ms": round(t_upd, 3),
+            "muon_matrices": len(owned),
+            "ns_TFLOPs_reference_flop_count": round(flops5 / (t_upd * 1e-3) / 1e12, 1),
+            "note": "40 owner-layout layer buffers packed and unpacked (padded staging of uneven shards, zero-filled pad "
+            "tails counted as written bytes), AdamW on the 41M-element fp32 tail shard, Muon on every 4th matrix",
+        }
+        del mats5, pa, ga, ma, va
+        torch.cuda.empty_cache()
     if legs:
         result["legs"] = legs
 

@@ -29,6 +29,7 @@ from ..core.layout import ShardPlan
 from ..core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module
 from ..core.plans import contiguous_even_plan, fsdp2_chunk_plan
 from .flat_buffer import MatrixFlatBuffer
+from .grad_bucket import BucketParamGrad, MatrixGradBucket
 
 Planner = Callable[[list[ManagedParam], int], ShardPlan]
 
@@ -248,8 +249,6 @@ class MatrixFSDPParamGroup:
             if missing:
                 # parameters without a gradient contribute zeros, as a reduce-scatter of an untouched workspace would
                 zeros = [(mp, torch.zeros(mp.numel, dtype=bucket.param_grads[0].grad.dtype, device=fb.device)) for mp in missing]
-                from .grad_bucket import BucketParamGrad, MatrixGradBucket
-
                 by_fqn = {pg.managed_param.fqn: pg for pg in bucket.param_grads}
                 by_fqn.update({mp.fqn: BucketParamGrad(mp, z) for mp, z in zeros})
                 ordered = tuple(by_fqn[mp.fqn] for mp in self.managed_params)
