@@ -8,8 +8,29 @@ the reference's shard metadata and operator signatures.
 from .core.layout import LayoutSegment, ShardPlan, validate_shard_plan
 from .core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module, managed_params_from_named
 from .api import MixedPrecisionPolicy, fully_shard, matrix_fully_shard
-from .optim.wrapper import MatrixOptimizerConfig, MixedMuonAdamWOptimizer, configure_optimizer
+from .core.placement import MatrixShard
+from .core.state import MatrixShardedState
+from .optim.state import MatrixFSDPOptimizerStateManager
+from .optim.wrapper import MatrixFSDPOptimizer, MatrixOptimizerConfig, MixedMuonAdamWOptimizer, configure_optimizer
 from .runtime.param_group import FSDPLifecycleState, MatrixFSDPParamGroup
+from .checkpoint import (
+    get_model_state_dict,
+    get_optimizer_state_dict,
+    get_state_dict,
+    load_matrix_dcp,
+    load_matrix_dcp_full_state,
+    load_matrix_state_dict,
+    matrix_get_state_dict,
+    matrix_set_state_dict,
+    matrix_state_dict,
+    patch_model_state_dict,
+    patch_optimizer_state_dict,
+    save_matrix_dcp,
+    save_matrix_dcp_simulated_world,
+    set_model_state_dict,
+    set_optimizer_state_dict,
+    set_state_dict,
+)
 
 __all__ = [
     "LayoutSegment",
@@ -27,4 +48,24 @@ __all__ = [
     "configure_optimizer",
     "FSDPLifecycleState",
     "MatrixFSDPParamGroup",
+    "MatrixShard",
+    "MatrixShardedState",
+    "MatrixFSDPOptimizer",
+    "MatrixFSDPOptimizerStateManager",
+    "get_model_state_dict",
+    "get_optimizer_state_dict",
+    "get_state_dict",
+    "load_matrix_dcp",
+    "load_matrix_dcp_full_state",
+    "load_matrix_state_dict",
+    "matrix_get_state_dict",
+    "matrix_set_state_dict",
+    "matrix_state_dict",
+    "patch_model_state_dict",
+    "patch_optimizer_state_dict",
+    "save_matrix_dcp",
+    "save_matrix_dcp_simulated_world",
+    "set_model_state_dict",
+    "set_optimizer_state_dict",
+    "set_state_dict",
 ]

@@ -122,3 +122,111 @@ def validate_shard_plan(plan: ShardPlan) -> None:
         cursor = end
     if cursor != plan.total_numel:
         raise ValueError(f"segments cover {cursor} of {plan.total_numel} elements.")
+
+
+# ---------------------------------------------------------------------------
+# Per-parameter view of a plan: what checkpoint metadata records.
+
+
+@dataclass(frozen=True)
+class ParamSegment:
+    """The part of parameter ``fqn`` inside one of rank ``rank``'s segments;
+    offsets as in ``LayoutSegment`` (matrix_fsdp/core/layout.py:33-55)."""
+
+    fqn: str
+    rank: int
+    global_start: int
+    global_end: int
+    local_start: int
+
+    @property
+    def numel(self) -> int:
+        return self.global_end - self.global_start
+
+    @property
+    def local_end(self) -> int:
+        return self.local_start + self.numel
+
+    def to_layout_segment(self) -> LayoutSegment:
+        return LayoutSegment(self.global_start, self.global_end, self.local_start)
+
+
+@dataclass(frozen=True)
+class RankLayout:
+    rank: int
+    local_units: int
+    segments: tuple[LayoutSegment, ...]
+
+
+@dataclass(frozen=True)
+class ParamLayout:
+    fqn: str
+    global_start: int
+    global_end: int
+    segments: tuple[ParamSegment, ...]
+
+    @property
+    def numel(self) -> int:
+        return self.global_end - self.global_start
+
+
+@dataclass(frozen=True)
+class MatrixGroupLayout:
+    """One unit's plan with the parameters cut along it
+    (matrix_fsdp/core/layout.py:100-211).  Offsets are flat-buffer offsets of
+    the unit, not of the model."""
+
+    total_numel: int
+    ranks: tuple[RankLayout, ...]
+    params: tuple[ParamLayout, ...] = ()
+
+    @classmethod
+    def from_rank_segments(cls, total_numel: int, rank_segments: RankSegments, params: tuple[ParamLayout, ...] = ()) -> "MatrixGroupLayout":
+        ranks = tuple(RankLayout(r, sum(s.numel for s in segs), tuple(segs)) for r, segs in enumerate(rank_segments))
+        return cls(total_numel, ranks, tuple(params))
+
+    @classmethod
+    def from_shard_plan(cls, plan: ShardPlan, params: Sequence = ()) -> "MatrixGroupLayout":
+        """``params`` are objects with ``fqn`` / ``offset`` / ``end``.  A
+        parameter's segments are listed rank by rank, and inside a rank in the
+        rank's segment order."""
+        param_layouts = []
+        for p in params:
+            pieces = []
+            for rank, segs in enumerate(plan.rank_segments):
+                for seg in segs:
+                    start, end = max(p.offset, seg.global_start), min(p.end, seg.global_end)
+                    if start < end:
+                        pieces.append(ParamSegment(p.fqn, rank, start, end, seg.local_start + start - seg.global_start))
+            param_layouts.append(ParamLayout(p.fqn, p.offset, p.end, tuple(pieces)))
+        return cls.from_rank_segments(plan.total_numel, plan.rank_segments, tuple(param_layouts))
+
+    @property
+    def world_size(self) -> int:
+        return len(self.ranks)
+
+    @property
+    def shard_sizes(self) -> tuple[int, ...]:
+        return tuple(rank.local_units for rank in self.ranks)
+
+    @property
+    def rank_segments(self) -> RankSegments:
+        return tuple(rank.segments for rank in self.ranks)
+
+    def param(self, fqn: str) -> ParamLayout:
+        for layout in self.params:
+            if layout.fqn == fqn:
+                return layout
+        raise KeyError(fqn)
+
+    def owner_ranks(self, fqn: str) -> tuple[int, ...]:
+        return tuple(sorted({seg.rank for seg in self.param(fqn).segments}))
+
+    def rank_segments_for_param(self, rank: int, fqn: str) -> tuple[ParamSegment, ...]:
+        return tuple(seg for seg in self.param(fqn).segments if seg.rank == rank)
+
+    def params_for_rank(self, rank: int) -> tuple[str, ...]:
+        return tuple(dict.fromkeys(seg.fqn for p in self.params for seg in p.segments if seg.rank == rank))
+
+    def to_shard_plan(self) -> ShardPlan:
+        return ShardPlan.from_rank_segments(self.total_numel, self.rank_segments)

@@ -234,6 +234,16 @@ def local_segments_program(segments, local_numel: int, output_numel: int, dtype:
     return SegmentProgram(make_runs(ls, gs, ln), (local_numel,), output_numel, src_dtype=dtype, device=device)
 
 
+def take_local_segments_program(segments, full_numel: int, local_numel: int, dtype: torch.dtype, *, out_dtype: torch.dtype | None = None, device="cuda") -> SegmentProgram:
+    """full flat buffer -> one rank's shard: the rank's row of ``pack_program``
+    on its own, as a checkpoint load into another layout needs it
+    (matrix_fsdp/checkpoint/state_dict.py:1330-1345)."""
+    gs = [s.global_start for s in segments]
+    ls = [s.local_start for s in segments]
+    ln = [s.global_end - s.global_start for s in segments]
+    return SegmentProgram(make_runs(gs, ls, ln), (full_numel,), local_numel, src_dtype=dtype, dst_dtype=out_dtype, device=device)
+
+
 def grad_fill_runs(params, rank_segments, max_shard: int) -> np.ndarray:
     """Runs of the generic copy-in: for every (rank, segment ∩ parameter) the
     slice of that parameter's grad goes to ``[rank, local_start + ...]`` of the

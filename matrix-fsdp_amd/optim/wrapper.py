@@ -21,6 +21,7 @@ from ..core.managed_param import ManagedParam
 from .adamw import FusedAdamW
 from .adamw_state import initialize_flat_adamw_state
 from .muon import Muon
+from .state import MatrixFSDPOptimizerStateManager
 
 DEFAULT_MUON_ADJUST_LR_FN = "match_rms_adamw"
 
@@ -58,6 +59,29 @@ def collect_flat_buffers(module_or_units) -> list:
             found.extend(getattr(module, "_matrix_fsdp_flat_buffers", ()))
         return found
     if hasattr(module_or_units, "local_param_views"):
+        return [module_or_units]
+    if hasattr(module_or_units, "flat_buffer"):  # one unit
+        return [] if module_or_units.flat_buffer is None else [module_or_units.flat_buffer]
+    found = []
+    for item in module_or_units:
+        buffer = getattr(item, "flat_buffer", item)  # a unit or a flat buffer
+        if buffer is not None:
+            found.append(buffer)
+    return found
+
+
+def collect_param_groups(module_or_units) -> list:
+    """The ``MatrixFSDPParamGroup`` units of a module (in ``named_modules``
+    order), of one unit, or of an iterable of units."""
+    if isinstance(module_or_units, nn.Module):
+        units, seen = [], set()
+        for module in module_or_units.modules():
+            unit = getattr(module, "_matrix_fsdp_param_group", None)
+            if unit is not None and id(unit) not in seen:
+                seen.add(id(unit))
+                units.append(unit)
+        return units
+    if hasattr(module_or_units, "flat_buffer"):
         return [module_or_units]
     return list(module_or_units)
 
@@ -284,3 +308,117 @@ def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig 
 
 
 configure_matrix_optimizer = configure_optimizer
+
+
+class MatrixFSDPOptimizer:
+    """An optimizer together with the units whose local parameters it steps:
+    the wrapper the reference hands to checkpointing
+    (matrix_fsdp/optim/wrapper.py:1002-1229).  On one device the units finish
+    their backward inside the autograd pass, so ``step`` has no lifecycle work
+    left; what remains is the opt-in flat AdamW state and the placement
+    metadata of the state tensors (``state_manager``).  The reference's
+    scheduler arguments have no counterpart and are not accepted."""
+
+    def __init__(self, optimizer, module_or_units, *, flat_adamw_state: bool = False) -> None:
+        self.optimizer = optimizer
+        self._fsdp_param_groups = collect_param_groups(module_or_units)
+        self.flat_adamw_state = flat_adamw_state
+        self.state_manager = MatrixFSDPOptimizerStateManager(optimizer, self._fsdp_param_groups)
+
+    @classmethod
+    def from_shard_hints(cls, module_or_units, *, default_matrix_optimizer: str = "muon", default_other_optimizer: str = "adamw", flat_adamw_state: bool = False, **optimizer_kwargs: Any) -> "MatrixFSDPOptimizer":
+        inner = make_mixed_muon_adamw_optimizer(
+            module_or_units,
+            default_matrix_optimizer=default_matrix_optimizer,
+            default_other_optimizer=default_other_optimizer,
+            flat_adamw_state=flat_adamw_state,
+            **optimizer_kwargs,
+        )
+        return cls(inner, module_or_units, flat_adamw_state=flat_adamw_state)
+
+    @property
+    def fsdp_param_groups(self) -> list:
+        return self._fsdp_param_groups
+
+    runtime_param_groups = fsdp_param_groups
+
+    @property
+    def param_groups(self) -> list[dict[str, Any]]:
+        return self.optimizer.param_groups
+
+    @property
+    def state(self) -> dict[Any, Any]:
+        return self.optimizer.state
+
+    @property
+    def defaults(self) -> dict[str, Any]:
+        return self.optimizer.defaults
+
+    def step(self, closure=None):
+        if closure is not None:
+            raise NotImplementedError("MatrixFSDPOptimizer V0 does not support optimizer closures.")
+        for unit in self._fsdp_param_groups:
+            unit.finalize_backward()  # a no-op once the autograd pass has finalised the unit
+        if self.flat_adamw_state and isinstance(self.optimizer, torch.optim.Optimizer):
+            initialize_flat_adamw_state(self.optimizer, collect_flat_buffers(self._fsdp_param_groups))
+        result = self.optimizer.step()
+        self.state_manager.refresh_state_dtensors()
+        return result
+
+    def zero_grad(self, *args: Any, **kwargs: Any) -> None:
+        self.optimizer.zero_grad(*args, **kwargs)
+
+    def state_dict(self) -> dict[str, Any]:
+        return self.optimizer.state_dict()
+
+    def load_state_dict(self, state_dict: dict[str, Any]) -> None:
+        self.optimizer.load_state_dict(state_dict)
+
+    def add_param_group(self, param_group: dict[str, Any]) -> None:
+        self.optimizer.add_param_group(param_group)
+
+    def optimizer_group_summary(self) -> dict[str, Any]:
+        """wrapper.py:1172-1195."""
+        if hasattr(self.optimizer, "optimizer_group_summary"):
+            return self.optimizer.optimizer_group_summary()
+        kind = type(self.optimizer).__name__
+        groups = []
+        for index, group in enumerate(self.optimizer.param_groups):
+            numel = sum(p.numel() for p in group["params"] if torch.is_tensor(p))
+            groups.append(
+                {
+                    "name": f"group_{index}",
+                    "optimizer_type": kind,
+                    "fqns": (),
+                    "num_params": sum(1 for p in group["params"] if torch.is_tensor(p)),
+                    "param_numel": numel,
+                    "local_numel": numel,
+                }
+            )
+        return {"optimizer": kind, "has_muon": False, "has_adamw": kind.lower().endswith("adamw"), "groups": tuple(groups)}
+
+    # ------------------------------------------------------------------ state placement metadata
+    def local_state_summary(self) -> dict[str, Any]:
+        return self.state_manager.local_state_summary()
+
+    def local_state_objects(self):
+        return self.state_manager.local_state_objects()
+
+    def local_state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.local_state_dtensors()
+
+    @property
+    def state_objects(self):
+        if not self.state_manager.state_objects:
+            self.state_manager.refresh_state_dtensors()
+        return self.state_manager.state_objects
+
+    @property
+    def state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.refresh_state_dtensors()
+
+    def refresh_state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.refresh_state_dtensors()
+
+    def validate_local_state_shapes(self) -> None:
+        self.state_manager.validate_local_state_shapes()

@@ -24,8 +24,16 @@ import torch
 
 from ..core.layout import LayoutSegment, ShardPlan, validate_shard_plan
 from ..core.managed_param import ManagedParam
+from ..core.placement import MatrixShard, explain_matrix_shard_compatibility, shard_sizes_to_matrix_local_units
+from ..core.state import MatrixShardedState
 from ..kernels import native
-from ..kernels.segment_program import SegmentProgram, compact_owner_program, pack_program, unpack_program
+from ..kernels.segment_program import (
+    SegmentProgram,
+    compact_owner_program,
+    pack_program,
+    take_local_segments_program,
+    unpack_program,
+)
 from .grad_bucket import (
     BucketParamGrad,
     CopyInBackend,
@@ -107,7 +115,62 @@ class MatrixFlatBuffer:
         self.grad_bucket_input: torch.Tensor | None = None
         self.grad_bucket_input_is_compact = False
         self.local_param_views = self._build_local_param_views()
+        # placement of the local shard in the flat buffer; plans a MatrixShard cannot express (several segments per
+        # rank) keep the shard sizes in lowest terms, as the reference does (flat_buffer.py:143-165)
+        self.matrix_shard_compatibility = explain_matrix_shard_compatibility(plan)
+        self.matrix_shard = MatrixShard((0,), shard_sizes_to_matrix_local_units(self.shard_sizes))
+        self.param_state = self._make_sharded_state("param", self.local_shard, self.matrix_shard, (plan.total_numel,))
         self.use_local_shards()
+
+    # ------------------------------------------------------------------ sharded-state metadata
+    @property
+    def local_numel(self) -> int:
+        return self.local_end - self.local_start
+
+    @property
+    def placement(self) -> MatrixShard:
+        return self.matrix_shard
+
+    @property
+    def grad_state(self) -> MatrixShardedState | None:
+        if self.local_grad_shard is None:
+            return None
+        return self._make_sharded_state("grad", self.local_grad_shard, self.matrix_shard, (self.plan.total_numel,))
+
+    def _make_sharded_state(self, name: str, local_tensor: torch.Tensor, placement: MatrixShard | None, global_shape: tuple[int, ...]) -> MatrixShardedState:
+        return MatrixShardedState(name, local_tensor, placement=placement, global_shape=global_shape, global_stride=(1,), requires_grad=local_tensor.requires_grad)
+
+    def param_shard_sizes(self, mp: ManagedParam) -> tuple[int, ...]:
+        """Elements of ``mp`` each rank holds (flat_buffer.py:1441-1451)."""
+        return tuple(
+            sum(max(0, min(mp.end, seg.global_end) - max(mp.offset, seg.global_start)) for seg in segments)
+            for segments in self.plan.rank_segments
+        )
+
+    def param_matrix_shard(self, mp: ManagedParam) -> MatrixShard | None:
+        """The parameter's own placement, when the ranks hold it as rank-ordered
+        contiguous pieces (flat_buffer.py:1433-1471)."""
+        cursor = 0
+        for segments in self.plan.rank_segments:
+            pieces = [(max(mp.offset, seg.global_start), min(mp.end, seg.global_end)) for seg in segments]
+            pieces = [(a - mp.offset, b - mp.offset) for a, b in pieces if a < b]
+            if not pieces:
+                continue
+            if len(pieces) != 1 or pieces[0][0] != cursor:
+                return None
+            cursor = pieces[0][1]
+        if cursor != mp.numel or mp.numel == 0:
+            return None
+        return MatrixShard((0,), shard_sizes_to_matrix_local_units(self.param_shard_sizes(mp)))
+
+    def make_param_state(self, mp: ManagedParam, name: str, local_tensor: torch.Tensor) -> MatrixShardedState | None:
+        """Metadata view of a shard-shaped tensor that belongs to ``mp`` (an
+        optimizer moment, say); ``None`` when the parameter has no placement
+        (flat_buffer.py:1417-1427)."""
+        placement = self.param_matrix_shard(mp)
+        if placement is None:
+            return None
+        return self._make_sharded_state(name, local_tensor.view(-1), placement, (mp.numel,))
 
     # ------------------------------------------------------------------ programs
     def _program(self, kind: str, dtype: torch.dtype, out_dtype: torch.dtype | None = None) -> SegmentProgram:
@@ -122,6 +185,10 @@ class MatrixFlatBuffer:
                 program = unpack_program(self.plan, dtype, padded=False, out_dtype=out_dtype, device=self.device)
             elif kind == "unpack_padded":
                 program = unpack_program(self.plan, dtype, padded=True, out_dtype=out_dtype, device=self.device)
+            elif kind == "take_local":
+                program = take_local_segments_program(
+                    self.local_segments, self.plan.total_numel, self.local_numel, dtype, out_dtype=out_dtype, device=self.device
+                )
             else:
                 raise KeyError(kind)
             self._programs[key] = program
@@ -224,6 +291,57 @@ class MatrixFlatBuffer:
         self.full_buffer = out
         self.use_full_param_buffer()
         return out
+
+    def gather_full_params(self) -> torch.Tensor:
+        """The full flat buffer in the local shard's dtype, assembled from the
+        current shards without touching ``param.data`` or ``full_buffer``
+        (what a checkpoint's ``full_state`` stores)."""
+        if self.world_shards is None:
+            raise RuntimeError("world shards were not kept; construct with keep_world_shards=True.")
+        return self._unpack_rank_shards_to_full_tensor(self.world_shards)
+
+    def gather_full_grads(self) -> torch.Tensor:
+        """The reduced gradient over the full flat buffer.  Only this rank's
+        gradient shard exists in a simulated world, so the other ranks' slots
+        are zero; with one rank this is the whole gradient."""
+        if self.local_grad_shard is None:
+            raise RuntimeError("Cannot build full gradients before local grad shard exists.")
+        packed = self.local_grad_shard.new_zeros(sum(self.shard_sizes))
+        if self.local_numel:
+            native.copy_range(self.local_grad_shard, packed[self.local_start : self.local_end], 0)
+        return self._unpack_rank_shards_to_full_tensor(packed)
+
+    def local_shard_from_full(self, full_tensor: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """This rank's shard of a full flat tensor, cast to the local dtype in
+        the same launch when the dtypes differ (bf16 <-> fp32 only)."""
+        full_tensor = full_tensor.reshape(-1)
+        if full_tensor.numel() != self.plan.total_numel:
+            raise ValueError(f"Full tensor has {full_tensor.numel()} elements, expected {self.plan.total_numel}.")
+        if out is None:
+            out = torch.empty(self.local_numel, dtype=self.local_shard.dtype, device=self.device)
+        if self.local_numel == 0:
+            return out
+        out_dtype = None if out.dtype == full_tensor.dtype else out.dtype
+        return self._program("take_local", full_tensor.dtype, out_dtype).run((full_tensor,), out)
+
+    def load_full_params(self, full_tensor: torch.Tensor) -> None:
+        """Re-shards a full flat tensor into this buffer: every simulated
+        rank's shard when the world is kept, else this rank's."""
+        full_tensor = full_tensor.reshape(-1)
+        if full_tensor.numel() != self.plan.total_numel:
+            raise ValueError(f"Full tensor has {full_tensor.numel()} elements, expected {self.plan.total_numel}.")
+        if self.world_shards is None:
+            self.local_shard_from_full(full_tensor, out=self.local_shard)
+            return
+        out_dtype = None if full_tensor.dtype == self.world_shards.dtype else self.world_shards.dtype
+        self._program("pack_compact", full_tensor.dtype, out_dtype).run((full_tensor,), self.world_shards)
+
+    def clear_full_params(self) -> None:
+        self.full_buffer = None
+
+    def clear_local_grad_shard(self) -> None:
+        self.local_grad_shard = None
+        self.grad_bucket_input = None
 
     def _pack_full_tensor_by_rank_segments(self, full_tensor: torch.Tensor) -> torch.Tensor:
         """flat_buffer.py:1304-1316."""
@@ -349,9 +467,13 @@ class MatrixFlatBuffer:
         self.local_grad_shard = self._maybe_to_local_dtype(chunk)
         return self.local_grad_shard
 
-    def use_local_grad_shard(self) -> None:
-        """``param.grad`` -> views of the reduced local grad shard
-        (flat_buffer.py:860-884)."""
+    def use_local_grad_shard(self, local_grad_shard: torch.Tensor | None = None) -> None:
+        """``param.grad`` -> views of the reduced local grad shard, which a
+        caller may hand in (flat_buffer.py:860-884)."""
+        if local_grad_shard is not None:
+            if local_grad_shard.numel() != self.local_numel:
+                raise ValueError(f"Local grad shard has {local_grad_shard.numel()} elements, expected {self.local_numel}.")
+            self.local_grad_shard = local_grad_shard.reshape(-1)
         if self.local_grad_shard is None:
             raise RuntimeError("Local gradient shard is not available.")
         by_param = self._local_views_by_param()

@@ -19,13 +19,14 @@ pointing into the reduced local gradient shard.
 from __future__ import annotations
 
 from enum import Enum
+from itertools import count
 from typing import Callable, Iterable, Mapping
 
 import torch
 from torch import nn
 from torch.autograd import Variable
 
-from ..core.layout import ShardPlan
+from ..core.layout import MatrixGroupLayout, ParamSegment, ShardPlan
 from ..core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module
 from ..core.plans import contiguous_even_plan, fsdp2_chunk_plan
 from .flat_buffer import MatrixFlatBuffer
@@ -34,6 +35,7 @@ from .grad_bucket import BucketParamGrad, MatrixGradBucket
 Planner = Callable[[list[ManagedParam], int], ShardPlan]
 
 _MANAGED_ATTR = "_matrix_fsdp_managed"
+_PARAM_GROUP_COUNTER = count()
 
 
 class FSDPLifecycleState(str, Enum):
@@ -107,6 +109,14 @@ class MatrixFSDPParamGroup:
         self.managed_params: list[ManagedParam] = []
         self.flat_buffer: MatrixFlatBuffer | None = None
         self.shard_plan: ShardPlan | None = None
+        self.group_layout: MatrixGroupLayout | None = None
+        # identifiers and mesh fields a checkpoint records (matrix_fsdp/runtime/runtime.py:47-53); one device has no
+        # mesh and no replicas
+        self.runtime_param_group_id = f"param_group_{next(_PARAM_GROUP_COUNTER)}"
+        self.replicate_world_size = 1
+        self.dp_shard_mesh_dim = 0
+        self.dp_replicate_mesh_dim = None
+        self.device_mesh_metadata = None
         self.lifecycle_state = FSDPLifecycleState.SHARDED
         self.events: list[str] = []
         self._handles: list = []
@@ -130,6 +140,7 @@ class MatrixFSDPParamGroup:
         if len(plan.shard_sizes) != self.world_size:
             raise ValueError(f"planner returned a plan for {len(plan.shard_sizes)} ranks, expected {self.world_size}.")
         self.shard_plan = plan
+        self.group_layout = MatrixGroupLayout.from_shard_plan(plan, self.managed_params)
         self.flat_buffer = MatrixFlatBuffer(
             self.managed_params, plan, self.rank, param_dtype=self.param_dtype, reduce_dtype=self.reduce_dtype
         )
@@ -147,6 +158,37 @@ class MatrixFSDPParamGroup:
         self.events.append(event)
         if len(self.events) > 256:
             del self.events[:128]
+
+    # ------------------------------------------------------------------ layout queries (fsdp_unit.py:822-850)
+    @property
+    def global_layout(self) -> MatrixGroupLayout | None:
+        """The planner's layout.  The unit runs the plan as it comes (several
+        segments per rank included), so it equals ``group_layout``: nothing is
+        flat-reordered."""
+        return self.group_layout
+
+    def owner_ranks(self, fqn: str) -> tuple[int, ...]:
+        return self.group_layout.owner_ranks(fqn)
+
+    def rank_segments_for_param(self, fqn: str, rank: int) -> tuple[ParamSegment, ...]:
+        return self.group_layout.rank_segments_for_param(rank, fqn)
+
+    def mixed_precision_metadata(self) -> dict[str, object]:
+        """matrix_fsdp/core/mixed_precision.py:11-17."""
+        name = lambda dtype: None if dtype is None else str(dtype)  # noqa: E731
+        return {
+            "param_dtype": name(self.param_dtype),
+            "reduce_dtype": name(self.reduce_dtype),
+            "output_dtype": name(self.output_dtype),
+            "cast_forward_inputs": bool(self.cast_forward_inputs),
+        }
+
+    def reset_after_load(self) -> None:
+        """A checkpoint load leaves the unit sharded with no backward pending."""
+        self.lifecycle_state = FSDPLifecycleState.SHARDED
+        self._seen_param_ids.clear()
+        self._backward_callback_queued = False
+        self._finalized_after_backward = True
 
     def remove_hooks(self) -> None:
         for handle in self._handles:
