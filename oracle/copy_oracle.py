@@ -14,7 +14,10 @@ Pinning (what makes this oracle trustworthy, see tests/test_oracle_*.py):
   * chunk-cat is checked against the library routine ``torch._chunk_cat``;
   * the 2x2 block layout is checked against the strided-slice closed form;
   * casts are checked against ``Tensor.to`` over crafted bit patterns;
-  * round trips and write-exactly-once invariants on random layouts.
+  * round trips and write-exactly-once invariants on random layouts;
+  * the checkpoint redistribution (``target_local_shard_from_full`` etc.) is
+    checked against the pinned pack / unpack functions: a rank's shard of the
+    full buffer is that rank's slice of the packed order, on random layouts.
 """
 from __future__ import annotations
 
@@ -350,3 +353,31 @@ def param_views(full: torch.Tensor, params) -> list[torch.Tensor]:
     """P5: ``full[offset:end].view(shape)`` per parameter, aliasing ``full``
     (matrix_fsdp/runtime/flat_buffer.py:413-425)."""
     return [full[p.offset : p.end].view(p.shape) for p in params]
+
+
+# ---------------------------------------------------------------- checkpoint load into another layout
+def target_local_shard_from_full(full: torch.Tensor, local_segments) -> torch.Tensor:
+    """One rank's shard of a full flat tensor: its segments' slices, concatenated
+    in segment order (matrix_fsdp/checkpoint/state_dict.py:1330-1345)."""
+    if not local_segments:
+        return full.new_empty(0)
+    return torch.cat([full[seg.global_start : seg.global_end] for seg in local_segments])
+
+
+def target_local_param_tensor_from_full(full_param: torch.Tensor, param_segments, param_offset: int) -> torch.Tensor:
+    """One rank's part of a parameter-shaped tensor (an optimizer moment) given
+    flat over the whole parameter; ``param_segments`` are the rank's segments
+    of that parameter in flat-buffer coordinates
+    (matrix_fsdp/checkpoint/state_dict.py:1348-1363)."""
+    if not param_segments:
+        return full_param.new_empty(0)
+    return torch.cat([full_param[seg.global_start - param_offset : seg.global_end - param_offset] for seg in param_segments])
+
+
+def full_from_source_rank_shards(source_shards: list[torch.Tensor]) -> torch.Tensor:
+    """The reference's reassembly of a saved flat buffer: the source ranks'
+    shards concatenated in rank order (state_dict.py:934-939).  Equal to the
+    full buffer only when the saved layout is rank-ordered; otherwise the
+    packed order has to be unpacked along the saved segments
+    (``unpack_rank_shards_to_full_tensor``)."""
+    return torch.cat([shard.reshape(-1) for shard in source_shards])

@@ -35,6 +35,7 @@ from matrix_fsdp_amd.core.plans import contiguous_even_plan, fsdp2_chunk_plan, w
 from matrix_fsdp_amd.optim.adamw import FusedAdamW
 from matrix_fsdp_amd.optim.state import MatrixFSDPOptimizerStateManager
 from matrix_fsdp_amd.optim.wrapper import MatrixFSDPOptimizer
+from oracle import copy_oracle as CO
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -551,9 +552,8 @@ def test_dcp_load_into_another_layout(tmp_path, source_world, source_planner, ta
                 load_matrix_dcp(model, tmp_path, optimizer=optimizer)
         load_matrix_dcp(model, tmp_path, optimizer=optimizer, allow_reshard=True)
         assert unit.lifecycle_state == FSDPLifecycleState.SHARDED
-        want_local = torch.cat([full_param[s.global_start : s.global_end] for s in fb.local_segments]) if fb.local_segments else full_param[:0]
-        assert torch.equal(fb.local_shard, want_local)
-        assert torch.equal(fb.local_grad_shard, torch.cat([full_grad[s.global_start : s.global_end] for s in fb.local_segments]))
+        assert torch.equal(fb.local_shard, CO.target_local_shard_from_full(full_param, fb.local_segments))
+        assert torch.equal(fb.local_grad_shard, CO.target_local_shard_from_full(full_grad, fb.local_segments))
         assert torch.equal(fb.gather_full_params(), full_param)  # every simulated rank's shard was refilled
         assert optimizer.param_groups[0]["lr"] == 0.01
         seen = 0
@@ -562,7 +562,7 @@ def test_dcp_load_into_another_layout(tmp_path, source_world, source_planner, ta
             state = optimizer.state[mp.param]
             assert int(state["step"].item()) == 1
             for name in ("exp_avg", "exp_avg_sq"):
-                want = full_state[name][mp.offset + view.param_start : mp.offset + view.param_end]
+                want = CO.target_local_param_tensor_from_full(full_state[name][mp.offset : mp.end], unit.rank_segments_for_param(mp.fqn, rank), mp.offset)
                 assert state[name].shape == mp.param.shape and torch.equal(state[name].reshape(-1), want), (rank, mp.fqn, name)
             seen += 1
         assert seen == len([p for p in model.parameters() if p.numel()])
@@ -570,8 +570,7 @@ def test_dcp_load_into_another_layout(tmp_path, source_world, source_planner, ta
         wide_step(model, optimizer, seed=4)
         if rank == 0:
             wide_step(whole, whole_optimizer, seed=4)
-        want_local = torch.cat([whole_fb.local_shard[s.global_start : s.global_end] for s in fb.local_segments])
-        assert torch.equal(fb.local_shard, want_local)
+        assert torch.equal(fb.local_shard, CO.target_local_shard_from_full(whole_fb.local_shard, fb.local_segments))
 
 
 def test_dcp_owner_layout_with_mixed_optimizer_into_another_world(tmp_path):

@@ -219,6 +219,40 @@ def test_round_trip_and_write_once_on_random_layouts():
         assert torch.equal(O.unpack_from_padded(padded, plan), full)
 
 
+def test_checkpoint_redistribution_on_random_layouts():
+    """A rank's shard of the full buffer is that rank's slice of the packed order; the reference's
+    concatenation of source shards is the full buffer exactly when the layout is rank-ordered, and the unpack is in
+    every case; a parameter's local part is the matching piece of the rank's shard."""
+    rng = random.Random(1)
+    ordered = 0
+    for _ in range(60):
+        total, world = rng.randint(2, 200), rng.randint(1, 5)
+        plan = random_plan(rng, total, world) if rng.random() < 0.7 else contiguous_even_plan(total, world)
+        full = torch.randperm(total).float() + 1
+        packed = O.pack_full_tensor_by_rank_segments(full, plan)
+        shards = []
+        for rank in range(world):
+            start = O.rank_packed_offset(plan.shard_sizes, rank)
+            shard = O.target_local_shard_from_full(full, plan.rank_segments[rank])
+            assert torch.equal(shard, packed[start : start + plan.shard_sizes[rank]])
+            shards.append(shard)
+        joined = O.full_from_source_rank_shards(shards)
+        assert torch.equal(joined, packed)
+        assert torch.equal(joined, full) == O.packed_rank_shards_are_full_tensor_order(plan)
+        ordered += int(torch.equal(joined, full))
+        assert torch.equal(O.unpack_rank_shards_to_full_tensor(joined, plan), full)
+        # a "parameter" [a, b) of the flat buffer and a moment tensor over it
+        a = rng.randint(0, total - 1)
+        b = rng.randint(a + 1, total)
+        moment = full[a:b] * 2
+        for rank in range(world):
+            pieces = [type(seg)(max(a, seg.global_start), min(b, seg.global_end), 0) for seg in plan.rank_segments[rank] if max(a, seg.global_start) < min(b, seg.global_end)]
+            local = O.target_local_param_tensor_from_full(moment, pieces, a)
+            want = torch.cat([shards[rank][seg.local_start + max(a, seg.global_start) - seg.global_start : seg.local_start + min(b, seg.global_end) - seg.global_start] for seg in plan.rank_segments[rank] if max(a, seg.global_start) < min(b, seg.global_end)] or [full.new_empty(0)])
+            assert torch.equal(local, want * 2)
+    assert 0 < ordered < 60  # both kinds of layout occurred
+
+
 def test_even_plan_sizes():
     plan = contiguous_even_plan(10, 4)
     assert plan.shard_sizes == (3, 3, 2, 2) and plan.shard_offsets == (0, 3, 6, 8)
