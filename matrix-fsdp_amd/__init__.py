@@ -11,6 +11,7 @@ from .api import MixedPrecisionPolicy, fully_shard, matrix_fully_shard
 from .core.placement import MatrixShard
 from .core.state import MatrixShardedState
 from .optim.state import MatrixFSDPOptimizerStateManager
+from .policy.wrap import and_policy, module_type_policy, not_policy, or_policy, size_based_policy
 from .optim.wrapper import MatrixFSDPOptimizer, MatrixOptimizerConfig, MixedMuonAdamWOptimizer, configure_optimizer
 from .runtime.param_group import FSDPLifecycleState, MatrixFSDPParamGroup
 from .checkpoint import (
@@ -52,6 +53,11 @@ __all__ = [
     "MatrixShardedState",
     "MatrixFSDPOptimizer",
     "MatrixFSDPOptimizerStateManager",
+    "and_policy",
+    "module_type_policy",
+    "not_policy",
+    "or_policy",
+    "size_based_policy",
     "get_model_state_dict",
     "get_optimizer_state_dict",
     "get_state_dict",

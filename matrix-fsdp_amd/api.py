@@ -19,6 +19,7 @@ from .core.layout import ShardPlan
 from .core.managed_param import ManagedParam, ParamShardHint
 from .planning.owner_plans import MuonOwnerPlanner
 from .planning.shard_hint import build_shard_hints
+from .policy.wrap import WrapPolicy
 from .runtime.param_group import MatrixFSDPParamGroup
 
 # optimizer_policy values of fully_shard (matrix_fsdp/api.py:43-54)
@@ -56,20 +57,33 @@ def matrix_fully_shard(
     ignored_params: set[nn.Parameter] | None = None,
     reshard_after_forward: bool = True,
     mp_policy=_DEFAULT_MP_POLICY,
+    wrap_policy: WrapPolicy | None = None,
+    auto_shard_hints: bool = False,
+    auto_planner_policy: str | None = None,
 ) -> nn.Module:
     """Turns ``module`` into one unit: its parameters (those no nested unit
     manages yet) move into a flat buffer sharded by ``planner`` for the
     simulated world, become views of rank ``rank``'s local shard, and forward /
-    backward hooks unshard and reshard them.  Returns ``module``."""
+    backward hooks unshard and reshard them.  Returns ``module``.
+
+    With ``wrap_policy`` the module tree is walked from the top: a module the
+    policy selects becomes a unit (and is not descended into), the others'
+    own parameters stay unmanaged (matrix_fsdp/api.py:309-378, 505-624).
+    ``auto_shard_hints`` derives the hints from the module structure;
+    ``auto_planner_policy="muon_shard_aware"`` keeps every parameter whole on
+    an owner rank (the other planner families of the reference do not exist
+    here)."""
     validate_mixed_precision_policy(mp_policy)
-    if getattr(module, "_matrix_fsdp_param_group", None) is not None:
-        raise ValueError("module is already wrapped by matrix_fully_shard().")
-    MatrixFSDPParamGroup(
-        module,
+    if auto_planner_policy is not None:
+        if str(auto_planner_policy).lower() != "muon_shard_aware":
+            raise ValueError(f"auto_planner_policy={auto_planner_policy!r} is not available; only 'muon_shard_aware' is.")
+        if planner is not None:
+            raise ValueError("Pass either auto_planner_policy or an explicit planner, not both.")
+        planner = MuonOwnerPlanner()  # one object for every unit of this call: ranks are balanced across the units
+    unit_args = dict(
         world_size=world_size,
         rank=rank,
         planner=planner,
-        shard_hints=shard_hints,
         ignored_params=ignored_params,
         reshard_after_forward=reshard_after_forward,
         param_dtype=getattr(mp_policy, "param_dtype", None),
@@ -77,7 +91,39 @@ def matrix_fully_shard(
         output_dtype=getattr(mp_policy, "output_dtype", None),
         cast_forward_inputs=getattr(mp_policy, "cast_forward_inputs", True),
     )
+    if wrap_policy is not None:
+        if shard_hints is not None:
+            raise ValueError("wrap_policy does not support explicit shard_hints yet.")
+        if _wrap_selected(module, wrap_policy, ignored_params, auto_shard_hints, unit_args) == 0:
+            raise ValueError("wrap_policy did not select any modules to shard.")
+        return module
+    _make_unit(module, shard_hints, ignored_params, auto_shard_hints, unit_args)
     return module
+
+
+def _own_hints(module: nn.Module, ignored_params: set[nn.Parameter] | None) -> dict[str, ParamShardHint]:
+    """Structure-derived hints for the parameters this unit will manage."""
+    skip = {id(p) for p in ignored_params or ()}
+    mine = {fqn for fqn, p in module.named_parameters() if id(p) not in skip and not getattr(p, "_matrix_fsdp_managed", False)}
+    return {fqn: hint for fqn, hint in build_shard_hints(module).items() if fqn in mine}
+
+
+def _make_unit(module, shard_hints, ignored_params, auto_shard_hints: bool, unit_args: dict) -> None:
+    if getattr(module, "_matrix_fsdp_param_group", None) is not None:
+        raise ValueError("module is already wrapped by matrix_fully_shard().")
+    if auto_shard_hints and shard_hints is None:
+        shard_hints = _own_hints(module, ignored_params) or None
+    MatrixFSDPParamGroup(module, shard_hints=shard_hints, **unit_args)
+
+
+def _wrap_selected(module: nn.Module, wrap_policy: WrapPolicy, ignored_params, auto_shard_hints: bool, unit_args: dict) -> int:
+    if wrap_policy(module):
+        skip = {id(p) for p in ignored_params or ()}
+        if not any(id(p) not in skip for p in module.parameters()):
+            return 0
+        _make_unit(module, None, ignored_params, auto_shard_hints, unit_args)
+        return 1
+    return sum(_wrap_selected(child, wrap_policy, ignored_params, auto_shard_hints, unit_args) for child in module.children())
 
 
 def fully_shard(
@@ -105,9 +151,7 @@ def fully_shard(
         if policy in _MUON_OPTIMIZER_POLICIES:
             if shard_placement_fn is not None:
                 raise ValueError("fully_shard optimizer_policy cannot be combined with shard_placement_fn.")
-            skip = {id(p) for p in ignored_params or ()}
-            mine = {fqn for fqn, p in module.named_parameters() if id(p) not in skip and not getattr(p, "_matrix_fsdp_managed", False)}
-            hints = {fqn: hint for fqn, hint in build_shard_hints(module).items() if fqn in mine}
+            hints = _own_hints(module, ignored_params)
             planner = planner or MuonOwnerPlanner()
         elif policy not in _NOOP_OPTIMIZER_POLICIES:
             allowed = sorted(_MUON_OPTIMIZER_POLICIES | _NOOP_OPTIMIZER_POLICIES)

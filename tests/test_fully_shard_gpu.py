@@ -101,6 +101,40 @@ def test_single_rank_adamw_training_matches_eager():
         assert rel(have[name], want[name]) < 2e-6, name
 
 
+def test_wrap_policy_units_train_like_eager():
+    """``wrap_policy`` picks the blocks and the head as units (top-down, a selected module is not descended into);
+    with ``auto_shard_hints`` and the owner planner the matrices go to Muon."""
+    from matrix_fsdp_amd import matrix_fully_shard
+    from matrix_fsdp_amd.policy import module_type_policy, or_policy, size_based_policy
+
+    model, twin = make_pair(seed=3)
+    policy = or_policy(module_type_policy(Block), size_based_policy(64 * 16))  # Block would also pass the size test via its Linears, but is taken whole
+    assert matrix_fully_shard(model, wrap_policy=policy, auto_shard_hints=True, auto_planner_policy="muon_shard_aware") is model
+    units = {name: m._matrix_fsdp_param_group for name, m in model.named_modules() if hasattr(m, "_matrix_fsdp_param_group")}
+    assert sorted(units) == ["blocks.0", "blocks.1", "head"]
+    assert [len(u.managed_params) for u in units.values()] == [5, 5, 2]
+    assert len({id(u.planner) for u in units.values()}) == 1  # one owner planner balances the ranks across the units
+    assert units["blocks.0"].managed_params[2].shard_hint.optimizer_type == "muon"  # up.weight
+    opt = configure_optimizer(model, "mixed_muon_adamw", lr=2e-3, weight_decay=0.05)
+    muon_names = {fqn for g in opt.optimizer_group_summary()["groups"] if g["optimizer_type"] == "muon" for fqn in g["param_fqns"]}
+    assert muon_names == {"up.weight", "down.weight", "weight"}
+    matrices = [p for p in twin.parameters() if p.ndim == 2]
+    others = [p for p in twin.parameters() if p.ndim != 2]
+    defaults = opt.defaults
+    ref_muon = torch.optim.Muon(matrices, **{k: defaults["muon"][k] for k in ("lr", "weight_decay", "momentum", "nesterov", "ns_coefficients", "eps", "ns_steps", "adjust_lr_fn")})
+    ref_adamw = torch.optim.AdamW(others, **{k: defaults["adamw"][k] for k in ("lr", "betas", "eps", "weight_decay")}, foreach=False)
+    start = named_full_params(twin)
+    (x, y), = batches(1, seed=6)
+    torch.nn.functional.mse_loss(model(x), y).backward()
+    opt.step()
+    torch.nn.functional.mse_loss(twin(x), y).backward()
+    ref_muon.step()
+    ref_adamw.step()
+    have, want = named_full_params(model), named_full_params(twin)
+    for name in want:
+        assert rel(have[name] - start[name], want[name] - start[name]) < (1e-2 if want[name].ndim == 2 else 1e-5), name
+
+
 def test_single_rank_mixed_muon_adamw_training_matches_eager():
     model, twin = make_pair(seed=2)
     shard_all(model, reshard_after_forward=False)

@@ -225,3 +225,53 @@ def test_fully_shard_host_rules():
         validate_mixed_precision_policy(MixedPrecisionPolicy(reduce_dtype=torch.int64))
     with pytest.raises(TypeError, match="ParamShardHint"):
         fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: "muon")
+    # wrap policies decide before anything touches the device
+    from matrix_fsdp_amd import matrix_fully_shard
+    from matrix_fsdp_amd.policy import module_type_policy
+
+    with pytest.raises(ValueError, match="did not select any modules"):
+        matrix_fully_shard(torch.nn.Sequential(torch.nn.ReLU(), torch.nn.Tanh()), wrap_policy=module_type_policy(torch.nn.Linear))
+    with pytest.raises(ValueError, match="did not select any modules"):  # selected, but all of its parameters are ignored
+        lin = torch.nn.Linear(2, 2)
+        matrix_fully_shard(torch.nn.Sequential(lin), wrap_policy=module_type_policy(torch.nn.Linear), ignored_params=set(lin.parameters()))
+    with pytest.raises(ValueError, match="explicit shard_hints"):
+        matrix_fully_shard(module, wrap_policy=module_type_policy(torch.nn.Linear), shard_hints={})
+    with pytest.raises(ValueError, match="only 'muon_shard_aware'"):
+        matrix_fully_shard(module, auto_planner_policy="balanced")
+    with pytest.raises(ValueError, match="not both"):
+        matrix_fully_shard(module, auto_planner_policy="muon_shard_aware", planner=default_planner)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        matrix_fully_shard(module, wrap_policy=module_type_policy(torch.nn.Linear))
+
+
+def test_wrap_policies():
+    """The expectations of the reference's test/fsdp/test_wrap.py:9-65."""
+    from torch import nn
+
+    from matrix_fsdp_amd.policy import and_policy, module_type_policy, not_policy, or_policy, size_based_policy
+
+    assert module_type_policy(nn.Linear)(nn.Linear(4, 2)) and not module_type_policy(nn.Linear)(nn.ReLU())
+    both = module_type_policy({nn.Linear, nn.LayerNorm})
+    assert both(nn.Linear(4, 2)) and both(nn.LayerNorm(4)) and not both(nn.ReLU())
+    with pytest.raises(ValueError, match="at least one"):
+        module_type_policy(set())
+    with pytest.raises(TypeError, match="nn.Module types"):
+        module_type_policy({nn.Linear, object})
+    module = nn.Sequential(nn.Linear(4, 8), nn.ReLU(), nn.Linear(8, 2))
+    assert not size_based_policy(1)(module) and size_based_policy(1)(module[0])  # own parameters only by default
+    total = sum(p.numel() for p in module.parameters())
+    assert size_based_policy(total, recurse=True)(module) and not size_based_policy(total + 1, recurse=True)(module)
+    with pytest.raises(ValueError, match="non-negative"):
+        size_based_policy(-1)
+    linear, large = module_type_policy(nn.Linear), size_based_policy(32)
+    assert or_policy(linear, module_type_policy(nn.LayerNorm))(nn.Linear(4, 2))
+    assert not or_policy(module_type_policy(nn.LayerNorm), module_type_policy(nn.ReLU))(nn.Linear(4, 2))
+    assert and_policy(linear, large)(nn.Linear(4, 8)) and not and_policy(linear, large)(nn.Linear(2, 2))
+    assert not_policy(large)(nn.Linear(2, 2))
+    for make in (or_policy, and_policy):
+        with pytest.raises(ValueError, match="at least one"):
+            make()
+        with pytest.raises(TypeError, match="callable"):
+            make(linear, object())
+    with pytest.raises(TypeError, match="callable"):
+        not_policy(object())
