@@ -40,6 +40,8 @@ extern "C" {
 #define MFSDP_CONVERT_NONE 0         /* raw element move, any elem_bytes */
 #define MFSDP_CONVERT_BF16_TO_F32 1  /* exact widening (Tensor.to(float32)) */
 #define MFSDP_CONVERT_F32_TO_BF16 2  /* round-to-nearest-even, NaN -> 0x7FC0 (Tensor.to(bfloat16)) */
+#define MFSDP_CONVERT_F16_TO_F32 3   /* exact widening, fp16 denormals included (Tensor.to(float32)) */
+#define MFSDP_CONVERT_F32_TO_F16 4   /* round-to-nearest-even, NaN -> sign | 0x7E00 (Tensor.to(float16)) */
 
 const char* mfsdp_last_error(void);
 /* ABI version of the library; bumped on any signature change. */
@@ -116,7 +118,8 @@ int64_t mfsdp_merge_segment_runs(const mfsdp_copy_run* segs, int64_t n_segs, mfs
  * Validates the runs against the extents (src_numels[n_srcs], dst_numel),
  * compiles and uploads them.  Allocates device memory; synchronous.
  * `convert` is one of MFSDP_CONVERT_*; elem_bytes is the element size for
- * MFSDP_CONVERT_NONE (ignored otherwise: 2 -> 4 or 4 -> 2 bytes).
+ * MFSDP_CONVERT_NONE (ignored otherwise: 2 -> 4 or 4 -> 2 bytes: bf16 or fp16 on
+ * the 2-byte side).
  */
 int mfsdp_segment_program_create(const mfsdp_copy_run* runs, int64_t n_runs,
                                  const int64_t* src_numels, int32_t n_srcs, int64_t dst_numel,

@@ -16,6 +16,8 @@ OK = 0
 CONVERT_NONE = 0
 CONVERT_BF16_TO_F32 = 1
 CONVERT_F32_TO_BF16 = 2
+CONVERT_F16_TO_F32 = 3
+CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
 ABI_VERSION = 1

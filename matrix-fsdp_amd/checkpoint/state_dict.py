@@ -40,7 +40,7 @@ from torch import nn
 
 from ..core.layout import LayoutSegment, ShardPlan
 from ..kernels import native
-from ..kernels.segment_program import unpack_program
+from ..kernels.segment_program import CONVERTIBLE, unpack_program
 from ..optim.state import MatrixFSDPOptimizerStateManager
 from ..runtime.flat_buffer import MatrixFlatBuffer
 from ..runtime.param_group import MatrixFSDPParamGroup
@@ -265,7 +265,7 @@ def _into_local_dtype(fb: MatrixFlatBuffer, tensor: torch.Tensor) -> torch.Tenso
         tensor = tensor.to(fb.device)
     if tensor.dtype == fb.local_shard.dtype:
         return tensor
-    if {tensor.dtype, fb.local_shard.dtype} == {torch.bfloat16, torch.float32}:
+    if (tensor.dtype, fb.local_shard.dtype) in CONVERTIBLE:
         return native.cast(tensor.contiguous(), fb.local_shard.dtype)
     return tensor.to(fb.local_shard.dtype)
 

@@ -188,12 +188,6 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 32 * BK);
   };
-  auto multiply = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-  };
   // Software pipeline.  STAGES slabs are resident or in flight: the slab being multiplied and the next
   // STAGES - 1, streamed HBM -> LDS while the MFMAs run.  Fragments are double buffered in registers: the
   // TM + TN 128-bit LDS reads of step kk+1 are issued before the MFMAs of step kk (and waited for BEFORE the

@@ -130,9 +130,20 @@ __device__ __forceinline__ uint32_t f32_bits_to_bf16_bits(uint32_t u) {
   return ((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : rounded;
 }
 
-// SRC_B bytes in, DST_B bytes out.  Equal sizes: raw move.  DST_B = 2*SRC_B:
-// bf16 -> fp32.  SRC_B = 2*DST_B: fp32 -> bf16.
-template <int SRC_B, int DST_B>
+// fp16 <-> fp32 through the hardware conversions: widening is exact (fp16 denormals included), narrowing rounds to
+// nearest even (overflow to infinity, underflow through the fp16 denormals to zero); every NaN becomes the quiet NaN
+// 0x7E00 with its sign kept.
+__device__ __forceinline__ uint32_t f16_bits_to_f32_bits(uint32_t h) {
+  return __float_as_uint(static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h))));
+}
+__device__ __forceinline__ uint32_t f32_bits_to_f16_bits(uint32_t u) {
+  if ((u & 0x7fffffffu) > 0x7f800000u) return ((u >> 16) & 0x8000u) | 0x7e00u;
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(__uint_as_float(u)));
+}
+
+// SRC_B bytes in, DST_B bytes out.  Equal sizes: raw move.  DST_B = 2*SRC_B: bf16 (HALF: fp16) -> fp32.
+// SRC_B = 2*DST_B: fp32 -> bf16 (HALF: fp16).
+template <int SRC_B, int DST_B, bool HALF = false>
 __device__ __forceinline__ Words<DST_B> convert_group(const Words<SRC_B>& in) {
   Words<DST_B> out;
   if constexpr (SRC_B == DST_B) {
@@ -143,19 +154,20 @@ __device__ __forceinline__ Words<DST_B> convert_group(const Words<SRC_B>& in) {
 #pragma unroll
     for (int i = 0; i < n; ++i) {
       const uint32_t word = in.w[i / 2];
-      out.w[i] = (i & 1) ? (word & 0xffff0000u) : (word << 16);
+      if constexpr (HALF) out.w[i] = f16_bits_to_f32_bits((i & 1) ? (word >> 16) : (word & 0xffffu));
+      else out.w[i] = (i & 1) ? (word & 0xffff0000u) : (word << 16);
     }
   } else {
     constexpr int n = DST_B / 2;
 #pragma unroll
     for (int i = 0; i < (DST_B + 3) / 4; ++i) out.w[i] = 0;
 #pragma unroll
-    for (int i = 0; i < n; ++i) out.w[i / 2] |= f32_bits_to_bf16_bits(in.w[i]) << (16 * (i & 1));
+    for (int i = 0; i < n; ++i) out.w[i / 2] |= (HALF ? f32_bits_to_f16_bits(in.w[i]) : f32_bits_to_bf16_bits(in.w[i])) << (16 * (i & 1));
   }
   return out;
 }
 
-template <int SRC_B, int DST_B, int U, bool NT, bool NTS = NT>
+template <int SRC_B, int DST_B, int U, bool NT, bool NTS = NT, bool HALF = false>
 __global__ void __launch_bounds__(kBlockThreads)
 segment_program_kernel(SourceTable srcs, char* __restrict__ dst, const DevRun* __restrict__ runs,
                        const DevTile* __restrict__ tiles, uint32_t n_tiles) {
@@ -190,7 +202,7 @@ segment_program_kernel(SourceTable srcs, char* __restrict__ dst, const DevRun* _
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (live[u]) store_bytes<DST_B, NTS>(dst + doff[u] * DST_B, convert_group<SRC_B, DST_B>(data[u]));
+      if (live[u]) store_bytes<DST_B, NTS>(dst + doff[u] * DST_B, convert_group<SRC_B, DST_B, HALF>(data[u]));
     }
   }
 }
@@ -205,6 +217,8 @@ struct Tuning {
   int convert_group = 4;
 };
 Tuning g_tuning;
+
+bool is_half_conversion(int convert) { return convert == MFSDP_CONVERT_F16_TO_F32 || convert == MFSDP_CONVERT_F32_TO_F16; }
 
 // ---- host side -------------------------------------------------------------------------------
 
@@ -333,7 +347,7 @@ int compile_variant(mfsdp_segment_program* prog, int cap, std::vector<Compiled>*
   return MFSDP_OK;
 }
 
-template <int SRC_B, int DST_B>
+template <int SRC_B, int DST_B, bool HALF = false>
 int launch_one(const Compiled& c, const SourceTable& srcs, char* dst, hipStream_t stream) {
   const int cus = device_cu_count();
   const uint32_t want = (c.n_tiles + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -342,7 +356,7 @@ int launch_one(const Compiled& c, const SourceTable& srcs, char* dst, hipStream_
   const dim3 block(kBlockThreads);
   const int nt = g_tuning.nontemporal;  // 0 none, 1 loads and stores, 2 loads only, 3 stores only
 #define MFSDP_LAUNCH(U_, NTL_, NTS_)                                                                             \
-  hipLaunchKernelGGL((segment_program_kernel<SRC_B, DST_B, U_, NTL_, NTS_>), grid, block, 0, stream, srcs, dst, \
+  hipLaunchKernelGGL((segment_program_kernel<SRC_B, DST_B, U_, NTL_, NTS_, HALF>), grid, block, 0, stream, srcs, dst, \
                      c.runs, c.tiles, c.n_tiles)
 #define MFSDP_LAUNCH_NT(U_)                      \
   switch (nt) {                                  \
@@ -365,9 +379,13 @@ int launch_compiled(const mfsdp_segment_program* prog, const Compiled& c, const 
   const int db = c.group_units * prog->dst_unit;
 #define MFSDP_CASE(S_, D_) \
   if (sb == S_ && db == D_) return launch_one<S_, D_>(c, srcs, dst, stream)
+#define MFSDP_CONVERTING(S_, D_) \
+  if (sb == S_ && db == D_) return half ? launch_one<S_, D_, true>(c, srcs, dst, stream) : launch_one<S_, D_, false>(c, srcs, dst, stream)
+  const bool half = is_half_conversion(prog->convert);
   MFSDP_CASE(16, 16); MFSDP_CASE(8, 8); MFSDP_CASE(4, 4); MFSDP_CASE(2, 2); MFSDP_CASE(1, 1);
-  MFSDP_CASE(16, 32); MFSDP_CASE(8, 16); MFSDP_CASE(4, 8); MFSDP_CASE(2, 4);
-  MFSDP_CASE(32, 16); MFSDP_CASE(16, 8); MFSDP_CASE(8, 4); MFSDP_CASE(4, 2);
+  MFSDP_CONVERTING(16, 32); MFSDP_CONVERTING(8, 16); MFSDP_CONVERTING(4, 8); MFSDP_CONVERTING(2, 4);
+  MFSDP_CONVERTING(32, 16); MFSDP_CONVERTING(16, 8); MFSDP_CONVERTING(8, 4); MFSDP_CONVERTING(4, 2);
+#undef MFSDP_CONVERTING
 #undef MFSDP_CASE
   return fail(MFSDP_ERR_UNSUPPORTED, "no kernel for %d -> %d byte groups", sb, db);
 }
@@ -388,9 +406,11 @@ int setup_units(int convert, int elem_bytes, int* src_unit, int* dst_unit, int* 
       *src_unit = 1; *dst_unit = 1; *max_group = 16; *scale = elem_bytes;  // units are bytes
       return MFSDP_OK;
     case MFSDP_CONVERT_BF16_TO_F32:
+    case MFSDP_CONVERT_F16_TO_F32:
       *src_unit = 2; *dst_unit = 4; *max_group = g_tuning.convert_group; *scale = 1;
       return MFSDP_OK;
     case MFSDP_CONVERT_F32_TO_BF16:
+    case MFSDP_CONVERT_F32_TO_F16:
       *src_unit = 4; *dst_unit = 2; *max_group = g_tuning.convert_group; *scale = 1;
       return MFSDP_OK;
     default:
@@ -606,7 +626,7 @@ extern "C" int mfsdp_copy_rank_segments_to_full(const void* local, int64_t local
 namespace {
 
 // dst[g] = convert(src[g]) over n_groups contiguous vector groups, persistent grid-stride.
-template <int SRC_B, int DST_B, int U, bool NT>
+template <int SRC_B, int DST_B, int U, bool NT, bool HALF = false>
 __global__ void __launch_bounds__(kBlockThreads)
 linear_kernel(const char* __restrict__ src, char* __restrict__ dst, int64_t n_groups) {
   const int64_t span = static_cast<int64_t>(kBlockThreads) * U;
@@ -621,12 +641,12 @@ linear_kernel(const char* __restrict__ src, char* __restrict__ dst, int64_t n_gr
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t g = base + u * kBlockThreads + threadIdx.x;
-      if (g < n_groups) store_bytes<DST_B, NT>(dst + g * DST_B, convert_group<SRC_B, DST_B>(data[u]));
+      if (g < n_groups) store_bytes<DST_B, NT>(dst + g * DST_B, convert_group<SRC_B, DST_B, HALF>(data[u]));
     }
   }
 }
 
-template <int SRC_B, int DST_B>
+template <int SRC_B, int DST_B, bool HALF = false>
 int launch_linear(const char* src, char* dst, int64_t n_groups, hipStream_t stream) {
   if (n_groups <= 0) return MFSDP_OK;
   constexpr int U = 4;
@@ -635,9 +655,9 @@ int launch_linear(const char* src, char* dst, int64_t n_groups, hipStream_t stre
   const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.linear_blocks_per_cu);
   const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, cap))));
   if (g_tuning.nontemporal)
-    hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, true>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
+    hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, true, HALF>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
   else
-    hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, false>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
+    hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, false, HALF>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
   MFSDP_CHECK_LAUNCH("linear_kernel");
   return MFSDP_OK;
 }
@@ -645,7 +665,7 @@ int launch_linear(const char* src, char* dst, int64_t n_groups, hipStream_t stre
 // Moves `units` contiguous units: a wide body sized by the pointers' common alignment, then a
 // unit-wide tail for the remainder.
 int linear_dispatch(const char* src, char* dst, int64_t units, int src_unit, int dst_unit, int max_group,
-                    hipStream_t stream) {
+                    hipStream_t stream, bool half = false) {
   int g = std::min(pointer_alignment_units(src, src_unit, max_group), pointer_alignment_units(dst, dst_unit, max_group));
   const int64_t body = units / g;
   const int64_t tail = units - body * g;
@@ -653,17 +673,20 @@ int linear_dispatch(const char* src, char* dst, int64_t units, int src_unit, int
   int rc = MFSDP_ERR_UNSUPPORTED;
 #define MFSDP_CASE(S_, D_) \
   if (sb == S_ && db == D_) rc = launch_linear<S_, D_>(src, dst, body, stream)
+#define MFSDP_CONVERTING(S_, D_) \
+  if (sb == S_ && db == D_) rc = half ? launch_linear<S_, D_, true>(src, dst, body, stream) : launch_linear<S_, D_, false>(src, dst, body, stream)
   MFSDP_CASE(16, 16); MFSDP_CASE(8, 8); MFSDP_CASE(4, 4); MFSDP_CASE(2, 2); MFSDP_CASE(1, 1);
-  MFSDP_CASE(16, 32); MFSDP_CASE(8, 16); MFSDP_CASE(4, 8); MFSDP_CASE(2, 4);
-  MFSDP_CASE(32, 16); MFSDP_CASE(16, 8); MFSDP_CASE(8, 4); MFSDP_CASE(4, 2);
+  MFSDP_CONVERTING(16, 32); MFSDP_CONVERTING(8, 16); MFSDP_CONVERTING(4, 8); MFSDP_CONVERTING(2, 4);
+  MFSDP_CONVERTING(32, 16); MFSDP_CONVERTING(16, 8); MFSDP_CONVERTING(8, 4); MFSDP_CONVERTING(4, 2);
+#undef MFSDP_CONVERTING
 #undef MFSDP_CASE
   if (rc == MFSDP_ERR_UNSUPPORTED) return fail(rc, "no kernel for %d -> %d byte groups", sb, db);
   if (rc != MFSDP_OK || tail == 0) return rc;
   const char* ts = src + body * sb;
   char* td = dst + body * db;
   if (src_unit == 1) return launch_linear<1, 1>(ts, td, tail, stream);
-  if (src_unit == 2) return launch_linear<2, 4>(ts, td, tail, stream);
-  return launch_linear<4, 2>(ts, td, tail, stream);
+  if (src_unit == 2) return half ? launch_linear<2, 4, true>(ts, td, tail, stream) : launch_linear<2, 4, false>(ts, td, tail, stream);
+  return half ? launch_linear<4, 2, true>(ts, td, tail, stream) : launch_linear<4, 2, false>(ts, td, tail, stream);
 }
 
 }  // namespace
@@ -683,11 +706,11 @@ extern "C" int mfsdp_copy_range(const void* in, int64_t in_numel, void* out, int
 
 extern "C" int mfsdp_cast(const void* src, void* dst, int64_t numel, int convert, void* stream) {
   if (numel < 0) return fail(MFSDP_ERR_INVALID, "numel must be non-negative");
-  if (convert != MFSDP_CONVERT_BF16_TO_F32 && convert != MFSDP_CONVERT_F32_TO_BF16)
-    return fail(MFSDP_ERR_INVALID, "mfsdp_cast converts bf16->f32 or f32->bf16, got code %d", convert);
+  if (convert != MFSDP_CONVERT_BF16_TO_F32 && convert != MFSDP_CONVERT_F32_TO_BF16 && !is_half_conversion(convert))
+    return fail(MFSDP_ERR_INVALID, "mfsdp_cast converts bf16 / f16 -> f32 or f32 -> bf16 / f16, got code %d", convert);
   if (numel == 0) return MFSDP_OK;
   if (src == nullptr || dst == nullptr) return fail(MFSDP_ERR_INVALID, "src or dst is null");
-  const bool widen = convert == MFSDP_CONVERT_BF16_TO_F32;
+  const bool widen = convert == MFSDP_CONVERT_BF16_TO_F32 || convert == MFSDP_CONVERT_F16_TO_F32;
   return linear_dispatch(static_cast<const char*>(src), static_cast<char*>(dst), numel, widen ? 2 : 4, widen ? 4 : 2,
-                         g_tuning.convert_group, as_stream(stream));
+                         g_tuning.convert_group, as_stream(stream), is_half_conversion(convert));
 }

@@ -145,19 +145,23 @@ def copy_range(input_tensor: torch.Tensor, output_tensor: torch.Tensor, input_of
         )
 
 
+_CAST_CODES = {
+    (torch.bfloat16, torch.float32): _lib.CONVERT_BF16_TO_F32,
+    (torch.float32, torch.bfloat16): _lib.CONVERT_F32_TO_BF16,
+    (torch.float16, torch.float32): _lib.CONVERT_F16_TO_F32,
+    (torch.float32, torch.float16): _lib.CONVERT_F32_TO_F16,
+}
+
+
 def cast(source: torch.Tensor, dtype: torch.dtype, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``source.to(dtype)`` for bfloat16<->float32 on the HIP cast kernel;
+    """``source.to(dtype)`` for bfloat16 / float16 <-> float32 on the HIP cast kernel;
     returns ``source`` itself when nothing changes, as the reference's
     ``_maybe_to_*_dtype`` helpers do (runtime/flat_buffer.py:1186-1206)."""
     if source.dtype == dtype or not source.is_floating_point():
         return source
-    pair = (source.dtype, dtype)
-    if pair == (torch.bfloat16, torch.float32):
-        code = _lib.CONVERT_BF16_TO_F32
-    elif pair == (torch.float32, torch.bfloat16):
-        code = _lib.CONVERT_F32_TO_BF16
-    else:
-        raise RuntimeError(f"HIP cast supports bfloat16<->float32, got {source.dtype} -> {dtype}")
+    code = _CAST_CODES.get((source.dtype, dtype))
+    if code is None:
+        raise RuntimeError(f"HIP cast supports bfloat16 / float16 <-> float32, got {source.dtype} -> {dtype}")
     if not source.is_cuda or not source.is_contiguous():
         raise RuntimeError("cast source must be a contiguous CUDA tensor")
     if out is None:

@@ -47,7 +47,10 @@ MAX_SOURCES = 128
 _CONVERT_CODES = {
     (torch.bfloat16, torch.float32): _lib.CONVERT_BF16_TO_F32,
     (torch.float32, torch.bfloat16): _lib.CONVERT_F32_TO_BF16,
+    (torch.float16, torch.float32): _lib.CONVERT_F16_TO_F32,
+    (torch.float32, torch.float16): _lib.CONVERT_F32_TO_F16,
 }
+CONVERTIBLE = frozenset(_CONVERT_CODES)  # (source dtype, destination dtype) pairs a program or a cast can convert
 
 
 def make_runs(src_off, dst_off, row_len, src_id=0) -> np.ndarray:
@@ -114,7 +117,7 @@ class SegmentProgram:
         elif (src_dtype, dst_dtype) in _CONVERT_CODES:
             convert, elem_bytes = _CONVERT_CODES[(src_dtype, dst_dtype)], 0
         else:
-            raise RuntimeError(f"segment programs convert bfloat16<->float32 only, got {src_dtype} -> {dst_dtype}.")
+            raise RuntimeError(f"segment programs convert bfloat16 / float16 <-> float32 only, got {src_dtype} -> {dst_dtype}.")
         if len(src_numels) > MAX_SOURCES:
             raise RuntimeError(f"a segment program reads at most {MAX_SOURCES} sources, got {len(src_numels)}.")
         self.src_dtype, self.dst_dtype = src_dtype, dst_dtype

@@ -313,7 +313,7 @@ class MatrixFlatBuffer:
 
     def local_shard_from_full(self, full_tensor: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """This rank's shard of a full flat tensor, cast to the local dtype in
-        the same launch when the dtypes differ (bf16 <-> fp32 only)."""
+        the same launch when the dtypes differ (bf16 or fp16 <-> fp32)."""
         full_tensor = full_tensor.reshape(-1)
         if full_tensor.numel() != self.plan.total_numel:
             raise ValueError(f"Full tensor has {full_tensor.numel()} elements, expected {self.plan.total_numel}.")

@@ -193,6 +193,55 @@ def test_cast_matches_tensor_to():
     assert native.cast(same, torch.float32) is same
 
 
+def test_fp16_casts_match_tensor_to():
+    """float16 <-> float32: every half bit pattern widened; narrowing at every rounding boundary (each finite half
+    value, the midpoint to its neighbour and one float32 step either side of it), around the overflow threshold,
+    through the denormal range, and on random bit patterns.  Numbers are bit-exact against ``Tensor.to`` on the
+    CPU; every NaN comes out as the quiet NaN 0x7E00 with its sign."""
+    all_half = torch.arange(-(2**15), 2**15, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    want = all_half.to(torch.float32)
+    have = native.cast(all_half.to(DEV), torch.float32).cpu()
+    numbers = ~torch.isnan(want)
+    assert torch.equal(have.view(torch.int32)[numbers], want.view(torch.int32)[numbers])
+    assert torch.isnan(have[~numbers]).all() and int(numbers.sum()) == 65536 - 2 * 1023
+
+    finite = want[torch.isfinite(want)].double().sort().values.unique()
+    mids = ((finite[:-1] + finite[1:]) / 2).float()  # exact: 12 significant bits
+    edge = torch.tensor([65504.0, 65519.99, 65520.0, 65520.01, 70000.0, 1e38, 2.0**-24, 2.0**-25, 2.0**-25 * 1.0000001, 2.0**-26, 1e-45, 0.0])
+    gen = torch.Generator().manual_seed(9)
+    random_bits = torch.randint(-(2**31), 2**31 - 1, (1 << 16,), generator=gen, dtype=torch.int64).to(torch.int32).view(torch.float32)
+    inf = torch.tensor(float("inf"))
+    x = torch.cat((finite.float(), mids, torch.nextafter(mids, inf), torch.nextafter(mids, -inf), edge, -edge, random_bits, torch.tensor([float("inf"), float("-inf")])))
+    for shift, n in ((0, x.numel()), (1, 4099), (3, 13), (0, 1)):
+        xs = x[shift : shift + n].contiguous()
+        have = native.cast(xs.to(DEV), torch.float16).cpu().view(torch.int16)
+        want16 = xs.to(torch.float16).view(torch.int16)
+        nan = torch.isnan(xs)
+        assert torch.equal(have[~nan], want16[~nan])
+        sign = (xs.view(torch.int32)[nan] >> 16) & -32768
+        assert torch.equal(have[nan].to(torch.int32) & 0xFFFF, (sign | 0x7E00) & 0xFFFF)
+    assert int(torch.isnan(x).sum()) > 0
+
+    # the same conversions folded into segment programs: fp16 grads into an fp32 workspace, fp32 shards gathered in fp16
+    rng = random.Random(3)
+    for _ in range(10):
+        world = rng.randint(1, 4)
+        sizes = [rng.randint(1, 500) for _ in range(rng.randint(1, 5))]
+        params = params_from_pairs([(f"p{i}", n) for i, n in enumerate(sizes)])
+        total = sum(sizes)
+        plan = random_plan(rng, total, world) if total > 1 else contiguous_even_plan(total, world)
+        grads_cpu = [torch.randn(n).half() for n in sizes]
+        expect = torch.full((world * plan.max_shard_size,), 3.0)
+        O.fill_reduce_scatter_input(params, grads_cpu, plan.shard_sizes, plan.rank_segments, total, expect)
+        packed = torch.full((world * plan.max_shard_size,), 5.0, device=DEV)
+        grad_fill_program(params, plan.shard_sizes, plan.rank_segments, torch.float16, torch.float32, device=DEV).run([g.to(DEV) for g in grads_cpu], packed)
+        assert_same_bits(packed, expect)
+        full = torch.randn(total) * 300
+        gathered = torch.empty(world * plan.max_shard_size, dtype=torch.float16, device=DEV)
+        pack_program(plan, torch.float32, out_dtype=torch.float16, device=DEV).run((full.to(DEV),), gathered)
+        assert torch.equal(gathered.cpu().view(torch.int16), O.pack_to_padded(full, plan).to(torch.float16).view(torch.int16))
+
+
 def test_random_layouts_every_width():
     rng = random.Random(1)
     for trial in range(40):

@@ -163,12 +163,13 @@ def test_single_rank_mixed_muon_adamw_training_matches_eager():
             assert rel(have[name] - start[name], want[name] - start[name]) < tol, (step, name)
 
 
-def test_mixed_precision_bf16_compute_fp32_master():
+@pytest.mark.parametrize("low", [torch.bfloat16, torch.float16])
+def test_mixed_precision_low_precision_compute_fp32_master(low):
     model, twin = make_pair(seed=3)
-    policy = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
+    policy = MixedPrecisionPolicy(param_dtype=low, reduce_dtype=torch.float32)
     for block in model.blocks:
         fully_shard(block, mp_policy=policy)
-    fully_shard(model, mp_policy=MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32, output_dtype=torch.float32))
+    fully_shard(model, mp_policy=MixedPrecisionPolicy(param_dtype=low, reduce_dtype=torch.float32, output_dtype=torch.float32))
     opt = configure_optimizer(model, "adamw", lr=1e-3, betas=(0.9, 0.95), weight_decay=0.0)
     ref = torch.optim.AdamW(twin.parameters(), lr=1e-3, betas=(0.9, 0.95), weight_decay=0.0, foreach=False)
     seen_dtypes = []
@@ -181,9 +182,9 @@ def test_mixed_precision_bf16_compute_fp32_master():
             fb = unit._matrix_fsdp_param_group.flat_buffer
             assert fb.local_shard.dtype == torch.float32 and fb.local_grad_shard.dtype == torch.float32
             assert all(mp.param.dtype == torch.float32 and mp.param.grad.dtype == torch.float32 for mp in fb.managed_params)
-        # eager twin: bf16 working copy of the fp32 master weights, grads cast up
-        work = copy.deepcopy(twin).bfloat16()
-        torch.nn.functional.mse_loss(work(x.bfloat16()).float(), y).backward()
+        # eager twin: low-precision working copy of the fp32 master weights, grads cast up
+        work = copy.deepcopy(twin).to(low)
+        torch.nn.functional.mse_loss(work(x.to(low)).float(), y).backward()
         for master, w in zip(twin.parameters(), work.parameters()):
             master.grad = w.grad.float()
         for (name, p), master in zip(model.named_parameters(), twin.parameters()):
@@ -192,7 +193,7 @@ def test_mixed_precision_bf16_compute_fp32_master():
         opt.zero_grad()
         ref.step()
         ref.zero_grad()
-    assert seen_dtypes and all(w == torch.bfloat16 and a == torch.bfloat16 for w, a in seen_dtypes)
+    assert seen_dtypes and all(w == low and a == low for w, a in seen_dtypes)
     have, want = named_full_params(model), named_full_params(twin)
     for name in want:
         assert rel(have[name], want[name]) < 2e-6, name
