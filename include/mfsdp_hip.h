@@ -184,8 +184,8 @@ int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t rows, int6
  * _adjust_lr(lr, fn, shape) (torch/optim/_muon.py:73-84).
  */
 int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols,
-                    float lr, float weight_decay, float momentum, int nesterov,
-                    float a, float b, float c, int steps, float eps, float adjusted_lr,
+                    double lr, double weight_decay, double momentum, int nesterov,
+                    float a, float b, float c, int steps, float eps, double adjusted_lr,
                     void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Kernel selection for experiments (values <= 0 keep the current setting):
@@ -203,11 +203,25 @@ void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direc
  * torch/optim/adam.py:347-547 with decoupled weight decay, reached through
  * matrix_fsdp/optim/wrapper.py:439, 497-516; state laid out flat as in
  * matrix_fsdp/optim/adamw_state.py:177-218).  `step` is the 1-based step
- * count after this update.  grad_dtype: MFSDP_F32 or MFSDP_BF16.
+ * count after this update.  grad_dtype: MFSDP_F32 or MFSDP_BF16.  The
+ * hyper-parameters are doubles, as Python holds them: 1 - beta, lr / (1 - beta1^t)
+ * and the like are formed in double and rounded to fp32 once, as torch does.
  */
 int mfsdp_adamw_step(float* param, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
-                     int64_t numel, int64_t step, float lr, float beta1, float beta2, float eps,
-                     float weight_decay, void* stream);
+                     int64_t numel, int64_t step, double lr, double beta1, double beta2, double eps,
+                     double weight_decay, void* stream);
+
+/*
+ * The same update with the two remaining switches of torch.optim.AdamW's
+ * single-tensor path (torch/optim/adam.py:398-399, 470-481): `maximize`
+ * negates the gradient; a non-null `max_exp_avg_sq` turns on amsgrad (the
+ * running element-wise maximum of the second moment, updated in place, takes
+ * the second moment's place in the denominator; the reference lays it out
+ * flat beside the moments, matrix_fsdp/optim/adamw_state.py:24-28).
+ */
+int mfsdp_adamw_step_ex(float* param, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
+                        float* max_exp_avg_sq, int64_t numel, int64_t step, double lr, double beta1, double beta2,
+                        double eps, double weight_decay, int maximize, void* stream);
 
 #ifdef __cplusplus
 }

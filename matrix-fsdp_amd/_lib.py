@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libmfsdp_hip.so")
@@ -65,13 +65,17 @@ SIGNATURES = {
     ),
     "mfsdp_muon_step": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_float, c_float, c_float, c_int,
-         c_float, c_float, c_float, c_int, c_float, c_float, c_void_p, c_int64, c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_double, c_double, c_double, c_int,
+         c_float, c_float, c_float, c_int, c_float, c_double, c_void_p, c_int64, c_void_p],
     ),
     "mfsdp_set_muon_tuning": (None, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "mfsdp_adamw_step": (
         c_int,
-        [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_float, c_float, c_float, c_float, c_float, c_void_p],
+        [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_double, c_double, c_double, c_double, c_double, c_void_p],
+    ),
+    "mfsdp_adamw_step_ex": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_double, c_double, c_double, c_double, c_double, c_int, c_void_p],
     ),
 }
 

@@ -134,31 +134,33 @@ extern "C" int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t
   if (!update || !out_bf16) return fail(MFSDP_ERR_INVALID, "null tensor pointer");
   hipStream_t s = as_stream(stream);
   int n_partials = 0;
-  if (int rc = muon_momentum(update, nullptr, update_dtype, rows * cols, 0.0f, 0, false, w.xraw, w.partials, &n_partials, s)) return rc;
+  if (int rc = muon_momentum(update, nullptr, update_dtype, rows * cols, 0.0, 0, false, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
   if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, &ortho, &ldo, s)) return rc;
   return muon_extract(out_bf16, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, s);
 }
 
-extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, float lr,
-                               float weight_decay, float momentum, int nesterov, float a, float b, float c, int steps, float eps,
-                               float adjusted_lr, void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, double lr,
+                               double weight_decay, double momentum, int nesterov, float a, float b, float c, int steps, float eps,
+                               double adjusted_lr, void* workspace, int64_t workspace_bytes, void* stream) {
   Workspace w;
   if (int rc = check_common(rows, cols, steps, workspace, workspace_bytes, &w)) return rc;
   if (dtype != MFSDP_F32 && dtype != MFSDP_BF16) return fail(MFSDP_ERR_INVALID, "dtype must be f32 or bf16");
   if (!param || !grad || !momentum_buf) return fail(MFSDP_ERR_INVALID, "null tensor pointer");
-  if (!(lr >= 0.0f)) return fail(MFSDP_ERR_INVALID, "Learning rate should be >= 0 but is: %g", lr);
-  if (!(momentum >= 0.0f)) return fail(MFSDP_ERR_INVALID, "momentum should be >= 0 but is: %g", momentum);
-  if (!(weight_decay >= 0.0f)) return fail(MFSDP_ERR_INVALID, "weight decay should be >= 0 but is: %g", weight_decay);
+  if (!(lr >= 0.0)) return fail(MFSDP_ERR_INVALID, "Learning rate should be >= 0 but is: %g", lr);
+  if (!(momentum >= 0.0)) return fail(MFSDP_ERR_INVALID, "momentum should be >= 0 but is: %g", momentum);
+  if (!(weight_decay >= 0.0)) return fail(MFSDP_ERR_INVALID, "weight decay should be >= 0 but is: %g", weight_decay);
   hipStream_t s = as_stream(stream);
   int n_partials = 0;
   if (int rc = muon_momentum(grad, momentum_buf, dtype, rows * cols, momentum, nesterov, true, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
   if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, &ortho, &ldo, s)) return rc;
-  const float decay = static_cast<float>(1.0 - static_cast<double>(lr) * static_cast<double>(weight_decay));
-  return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, decay, -adjusted_lr, s);
+  // the host scalars are doubles, as in Python: 1 - lr * wd and -adjusted_lr are rounded to fp32 once, where the
+  // tensor operation takes them
+  const float decay = static_cast<float>(1.0 - lr * weight_decay);
+  return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, decay, static_cast<float>(-adjusted_lr), s);
 }
 
 extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,

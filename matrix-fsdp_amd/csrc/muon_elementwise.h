@@ -11,7 +11,7 @@ constexpr int kMuonMaxPartials = 2048;
 
 // xraw <- bf16(u), partials <- per-block sums of bf16(u)^2, where u is the momentum/Nesterov update
 // (with_momentum; buf updated in place) or grad itself.  dtype: MFSDP_F32 / MFSDP_BF16 of grad and buf.
-int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, float momentum, int nesterov, bool with_momentum,
+int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, double momentum, int nesterov, bool with_momentum,
                   void* xraw, float* partials, int* n_partials, hipStream_t stream);
 // scalars[0] <- max(bf16(sqrt(sum partials)), bf16(eps))
 int muon_norm(const float* partials, int n_partials, float eps, float* scalars, hipStream_t stream);

@@ -26,8 +26,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 
 // Tensor.lerp as ATen evaluates it.
 __device__ __forceinline__ float lerp_aten(float start, float end, float weight) {
+  // one fused multiply-add from the nearer end point, the form ATen's vectorised kernel spells out
+  // (fmadd(weight, end - start, start) / fmadd(weight - 1, end - start, end)); written explicitly so that the
+  // compiler's contraction choices cannot differ between code paths
   const float diff = end - start;
-  return weight < 0.5f ? start + weight * diff : end - diff * (1.0f - weight);
+  return fabsf(weight) < 0.5f ? __builtin_fmaf(weight, diff, start) : __builtin_fmaf(weight - 1.0f, diff, end);
 }
 
 template <typename T>
@@ -151,7 +154,7 @@ norm_kernel(const float* __restrict__ partials, int n_partials, float eps, float
     __syncthreads();
   }
   if (threadIdx.x == 0) {
-    const float norm = bf16_to_f32(f32_to_bf16(__fsqrt_rn(static_cast<float>(lds[0]))));
+    const float norm = bf16_to_f32(f32_to_bf16(sqrtf(static_cast<float>(lds[0]))));
     const float floor_ = bf16_to_f32(f32_to_bf16(eps));
     scalars[0] = norm > floor_ ? norm : floor_;
   }
@@ -238,12 +241,13 @@ int partial_blocks(int64_t numel) {
 
 }  // namespace
 
-int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, float momentum, int nesterov, bool with_momentum,
+int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, double momentum, int nesterov, bool with_momentum,
                   void* xraw, float* partials, int* n_partials, hipStream_t stream) {
   const int blocks = partial_blocks(numel);
   *n_partials = blocks;
-  // the scalar the reference hands to lerp_ is the Python double 1 - momentum
-  const float one_minus = static_cast<float>(1.0 - static_cast<double>(momentum));
+  // the scalars torch hands to lerp_ are the Python doubles 1 - momentum and momentum, rounded to fp32 by the kernel
+  const float one_minus = static_cast<float>(1.0 - momentum);
+  const float weight = static_cast<float>(momentum);
   auto x = static_cast<uint16_t*>(xraw);
   const uintptr_t need = dtype == MFSDP_F32 ? 16 : 8;  // alignment of a group of four elements
   const bool aligned = reinterpret_cast<uintptr_t>(grad) % need == 0 && (!with_momentum || reinterpret_cast<uintptr_t>(buf) % need == 0) &&
@@ -252,13 +256,13 @@ int muon_momentum(const void* grad, void* buf, int dtype, int64_t numel, float m
   if (dtype == MFSDP_F32) {
     auto g = static_cast<const float*>(grad);
     auto b = static_cast<float*>(buf);
-    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<float, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
-    else hipLaunchKernelGGL((momentum_kernel<float, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<float, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, weight, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<float, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, weight, one_minus, nesterov);
   } else {
     auto g = static_cast<const uint16_t*>(grad);
     auto b = static_cast<uint16_t*>(buf);
-    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<uint16_t, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
-    else hipLaunchKernelGGL((momentum_kernel<uint16_t, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, momentum, one_minus, nesterov);
+    if (with_momentum) hipLaunchKernelGGL((momentum_kernel<uint16_t, true>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, weight, one_minus, nesterov);
+    else hipLaunchKernelGGL((momentum_kernel<uint16_t, false>), dim3(blocks), dim3(kThreads), 0, stream, g, b, x, partials, numel, n_quads, weight, one_minus, nesterov);
   }
   MFSDP_CHECK_LAUNCH("momentum_kernel");
   return MFSDP_OK;

@@ -1,7 +1,7 @@
 """``FusedAdamW``: AdamW on the HIP kernel, one launch per contiguous run of parameters.
 
 Hyper-parameters, parameter-group keys and state keys (``step``, ``exp_avg``,
-``exp_avg_sq``) are those of ``torch.optim.AdamW``, the optimizer the reference
+``exp_avg_sq``) are those of ``torch.optim.AdamW`` (``amsgrad`` and ``maximize`` included), the optimizer the reference
 builds for everything Muon does not take (matrix_fsdp/optim/wrapper.py:431-439);
 the arithmetic is the single-tensor path of torch/optim/adam.py:347-547.  When
 the parameters are views of one flat shard, their grads views of one local
@@ -42,17 +42,17 @@ class FusedAdamW(Optimizer):
             raise ValueError(f"Invalid beta parameter at index 1: {betas[1]}")
         if not 0.0 <= weight_decay:
             raise ValueError(f"Invalid weight_decay value: {weight_decay}")
-        if amsgrad or maximize:
-            raise NotImplementedError("FusedAdamW supports neither amsgrad nor maximize")
-        defaults = {"lr": lr, "betas": betas, "eps": eps, "weight_decay": weight_decay, "amsgrad": False, "maximize": False}
+        defaults = {"lr": lr, "betas": betas, "eps": eps, "weight_decay": weight_decay, "amsgrad": bool(amsgrad), "maximize": bool(maximize)}
         super().__init__(params, defaults)
 
-    def _init_state(self, p: Tensor) -> dict:
+    def _init_state(self, p: Tensor, amsgrad: bool) -> dict:
         state = self.state[p]
         if len(state) == 0:
             state["step"] = torch.tensor(0.0, dtype=torch.float32)
             state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
             state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            if amsgrad:
+                state["max_exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
         return state
 
     @torch.no_grad()
@@ -62,6 +62,7 @@ class FusedAdamW(Optimizer):
             with torch.enable_grad():
                 loss = closure()
         for group in self.param_groups:
+            amsgrad = bool(group.get("amsgrad", False))
             entries = []
             for p in group["params"]:
                 if p.grad is None or p.numel() == 0:
@@ -70,13 +71,17 @@ class FusedAdamW(Optimizer):
                     raise RuntimeError("AdamW does not support sparse gradients")
                 if p.dtype != torch.float32:
                     raise RuntimeError(f"FusedAdamW updates float32 parameters, got {p.dtype}")
-                state = self._init_state(p)
+                state = self._init_state(p, amsgrad)
                 state["step"] += 1
-                entries.append((p.data, p.grad.contiguous(), state["exp_avg"], state["exp_avg_sq"], int(state["step"].item())))
-            for param, grad, exp_avg, exp_avg_sq, step in _merge_contiguous(entries):
+                tensors = [p.data, p.grad.contiguous(), state["exp_avg"], state["exp_avg_sq"]]
+                if amsgrad:
+                    tensors.append(state["max_exp_avg_sq"])
+                entries.append((*tensors, int(state["step"].item())))
+            for *tensors, step in _merge_contiguous(entries):
                 F.adamw_step(
-                    param, grad, exp_avg, exp_avg_sq, step,
+                    *tensors[:4], step,
                     lr=group["lr"], betas=group["betas"], eps=group["eps"], weight_decay=group["weight_decay"],
+                    max_exp_avg_sq=tensors[4] if amsgrad else None, maximize=bool(group.get("maximize", False)),
                 )
         return loss
 
@@ -93,13 +98,13 @@ def _follows(prev: Tensor, nxt: Tensor) -> bool:
 
 
 def _merge_contiguous(entries):
-    """Merges neighbours whose parameter, grad and both moments each continue
-    the previous entry's memory inside one storage (and share a step count)
-    into one flat update.  Yields ``(param, grad, exp_avg, exp_avg_sq, step)``
+    """Merges neighbours whose parameter, grad and moments each continue the
+    previous entry's memory inside one storage (and share a step count) into
+    one flat update.  Yields ``(param, grad, exp_avg, exp_avg_sq[, max_exp_avg_sq], step)``
     as 1-D spans."""
     runs: list[dict] = []
     for tensors_and_step in sorted(entries, key=lambda e: e[0].data_ptr()):
-        tensors, step = tensors_and_step[:4], tensors_and_step[4]
+        tensors, step = tensors_and_step[:-1], tensors_and_step[-1]
         if runs:
             run = runs[-1]
             if run["step"] == step and all(_follows(a, b) for a, b in zip(run["last"], tensors)):

@@ -20,6 +20,7 @@ class FlatAdamWStateBuffers:
     total_numel: int
     exp_avg: torch.Tensor
     exp_avg_sq: torch.Tensor
+    max_exp_avg_sq: torch.Tensor | None = None  # with amsgrad
 
 
 def local_param_state_layout(flat_buffers) -> tuple[dict[int, tuple[int, int]], int]:
@@ -46,9 +47,10 @@ def local_param_state_layout(flat_buffers) -> tuple[dict[int, tuple[int, int]], 
 
 
 def initialize_flat_adamw_state(optimizer: Optimizer, flat_buffers) -> bool:
-    """Pre-creates ``state[p] = {step, exp_avg, exp_avg_sq}`` as views of flat
-    buffers for every parameter that has a grad and no state yet.  Returns
-    whether anything was initialised (matrix_fsdp/optim/adamw_state.py:44-87)."""
+    """Pre-creates ``state[p] = {step, exp_avg, exp_avg_sq[, max_exp_avg_sq]}``
+    as views of flat buffers for every parameter that has a grad and no state
+    yet.  Returns whether anything was initialised
+    (matrix_fsdp/optim/adamw_state.py:44-87, 133-175)."""
     spans, total = local_param_state_layout(flat_buffers)
     if not spans:
         return False
@@ -56,6 +58,7 @@ def initialize_flat_adamw_state(optimizer: Optimizer, flat_buffers) -> bool:
     optimizer._matrix_fsdp_flat_adamw_state_buffers = buffers
     initialised = False
     for group in optimizer.param_groups:
+        amsgrad = bool(group.get("amsgrad", False))
         for param in group["params"]:
             if param.grad is None or param.numel() == 0 or param.grad.is_sparse:
                 continue
@@ -76,10 +79,16 @@ def initialize_flat_adamw_state(optimizer: Optimizer, flat_buffers) -> bool:
                     f"Existing flat AdamW state has {buf.total_numel} elements, "
                     f"but the current MatrixFSDP optimizer layout expects {total}."
                 )
+            if amsgrad and buf.max_exp_avg_sq is None:
+                buf = buffers[key] = FlatAdamWStateBuffers(
+                    total, buf.exp_avg, buf.exp_avg_sq, torch.zeros(total, device=param.device, dtype=param.dtype)
+                )
             start, end = span
             state = optimizer.state[param]
             state["step"] = torch.tensor(0.0, dtype=torch.float32)
             state["exp_avg"] = buf.exp_avg[start:end].view_as(param)
             state["exp_avg_sq"] = buf.exp_avg_sq[start:end].view_as(param)
+            if amsgrad:
+                state["max_exp_avg_sq"] = buf.max_exp_avg_sq[start:end].view_as(param)
             initialised = True
     return initialised

@@ -146,10 +146,16 @@ def adamw_step(
     betas=(0.9, 0.999),
     eps: float = 1e-8,
     weight_decay: float = 1e-2,
+    max_exp_avg_sq: torch.Tensor | None = None,
+    maximize: bool = False,
 ) -> None:
     """Fused AdamW over flat fp32 tensors; ``step`` is the 1-based count after
-    this update (torch/optim/adam.py:347-547)."""
-    for t, what in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+    this update (torch/optim/adam.py:347-547).  ``max_exp_avg_sq`` turns on
+    amsgrad, ``maximize`` negates the gradient."""
+    state = [(param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")]
+    if max_exp_avg_sq is not None:
+        state.append((max_exp_avg_sq, "max_exp_avg_sq"))
+    for t, what in state:
         if not t.is_cuda or not t.is_contiguous() or t.dtype != torch.float32:
             raise RuntimeError(f"{what} must be a contiguous float32 CUDA tensor")
         if t.numel() != param.numel():
@@ -159,8 +165,9 @@ def adamw_step(
     stream = torch.cuda.current_stream(param.device).cuda_stream
     with torch.cuda.device(param.device):
         _lib.check(
-            _lib.lib().mfsdp_adamw_step(
+            _lib.lib().mfsdp_adamw_step_ex(
                 param.data_ptr(), grad.data_ptr(), _DTYPE_CODES[grad.dtype], exp_avg.data_ptr(), exp_avg_sq.data_ptr(),
-                param.numel(), int(step), lr, betas[0], betas[1], eps, weight_decay, stream,
+                None if max_exp_avg_sq is None else max_exp_avg_sq.data_ptr(),
+                param.numel(), int(step), lr, betas[0], betas[1], eps, weight_decay, int(bool(maximize)), stream,
             )
         )

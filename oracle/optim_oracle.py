@@ -105,16 +105,25 @@ def adamw_step(
     betas=(0.9, 0.999),
     eps: float = 1e-8,
     weight_decay: float = 1e-2,
+    max_exp_avg_sq: torch.Tensor | None = None,
+    maximize: bool = False,
 ) -> None:
     """Single-tensor AdamW, ``step`` being the 1-based count *after* this
-    update (torch/optim/adam.py:347-547: decoupled decay :417-419, moments
-    :457 and :476, bias corrections and the update :534-547)."""
+    update (torch/optim/adam.py:347-547: maximize :397, decoupled decay
+    :417-419, moments :457 and :476, bias corrections and the update :530-546
+    with the amsgrad maximum :537-541 when ``max_exp_avg_sq`` is given)."""
     beta1, beta2 = betas
+    if maximize:
+        grad = -grad
     param.mul_(1 - lr * weight_decay)
     exp_avg.lerp_(grad, 1 - beta1)
     exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
     bc1 = 1 - beta1**step
     bc2 = 1 - beta2**step
     step_size = lr / bc1
-    denom = (exp_avg_sq.sqrt() / math.sqrt(bc2)).add_(eps)
+    second = exp_avg_sq
+    if max_exp_avg_sq is not None:
+        torch.maximum(max_exp_avg_sq, exp_avg_sq, out=max_exp_avg_sq)
+        second = max_exp_avg_sq
+    denom = (second.sqrt() / math.sqrt(bc2)).add_(eps)
     param.addcdiv_(exp_avg, denom, value=-step_size)

@@ -464,6 +464,27 @@ def test_state_manager_describes_shard_shaped_state():
     assert summary.scalar_state_tensor_numel == 6 and summary.as_dict() == optimizer.local_state_summary()
     assert optimizer.state_objects and optimizer.state_dtensors == {} and optimizer.refresh_state_dtensors() == {}
 
+    # amsgrad: the running maximum is flat too, and the optimizer follows torch.optim.AdamW(amsgrad=True, maximize=True)
+    torch.manual_seed(0)
+    model = small_model()
+    twin = copy.deepcopy(model)
+    matrix_fully_shard(model)
+    optimizer = MatrixFSDPOptimizer(FusedAdamW(model.parameters(), lr=0.01, amsgrad=True, maximize=True), model, flat_adamw_state=True)
+    reference = torch.optim.AdamW(twin.parameters(), lr=0.01, amsgrad=True, maximize=True, foreach=False)
+    for seed in (7, 8, 9):
+        one_step(model, optimizer, seed=seed)
+        x = torch.randn(3, 4, generator=torch.Generator().manual_seed(seed)).to(DEV)
+        reference.zero_grad()
+        twin(x).sum().backward()
+        reference.step()
+    (flat,) = optimizer.optimizer._matrix_fsdp_flat_adamw_state_buffers.values()
+    assert flat.max_exp_avg_sq is not None and flat.max_exp_avg_sq.numel() == 58
+    states = [s for p, s in optimizer.optimizer.state.items() if p.numel()]
+    assert {s["max_exp_avg_sq"].untyped_storage().data_ptr() for s in states} == {flat.max_exp_avg_sq.untyped_storage().data_ptr()}
+    for have, want in zip(model.parameters(), twin.parameters()):
+        assert torch.allclose(have.detach(), want.detach(), rtol=0, atol=2e-6 * float(want.abs().max()))
+        assert torch.allclose(optimizer.state[have]["max_exp_avg_sq"], reference.state[want]["max_exp_avg_sq"], rtol=1e-5, atol=1e-10)
+
     # opt-in only
     torch.manual_seed(0)
     model = matrix_fully_shard(linear())

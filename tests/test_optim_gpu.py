@@ -132,6 +132,55 @@ def test_adamw_parity(n, grad_dtype):
         assert max_err_over_scale(v, v_cpu) < 1e-6
 
 
+@pytest.mark.parametrize("amsgrad,maximize", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("n", [1000, 4099])
+def test_adamw_amsgrad_and_maximize_parity(n, amsgrad, maximize):
+    p_cpu, m_cpu, v_cpu = make((n,), 5, 0.02), torch.zeros(n), torch.zeros(n)
+    x_cpu = torch.zeros(n) if amsgrad else None
+    p, m, v = p_cpu.to(DEV), m_cpu.to(DEV), v_cpu.to(DEV)
+    x = torch.zeros(n, device=DEV) if amsgrad else None
+    kw = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, maximize=maximize)
+    for t, scale in enumerate((1.0, 0.05, 0.2, 0.01), start=1):  # shrinking grads: the running maximum matters
+        g = make((n,), 30 + t) * scale
+        O.adamw_step(p_cpu, g, m_cpu, v_cpu, t, max_exp_avg_sq=x_cpu, **kw)
+        F.adamw_step(p, g.to(DEV), m, v, t, max_exp_avg_sq=x, **kw)
+        assert max_err_over_scale(p, p_cpu) < 1e-6
+        assert max_err_over_scale(m, m_cpu) < 1e-6
+        assert max_err_over_scale(v, v_cpu) < 1e-6
+        if amsgrad:
+            assert max_err_over_scale(x, x_cpu) < 1e-6
+    if amsgrad:
+        assert not torch.equal(x, v)
+
+
+def test_optimizer_scalars_are_formed_in_double():
+    """``1 - beta2`` for beta2 = 0.999 is 1.3e-5 off when it is formed from an fp32 beta2, and ``1 - momentum``
+    for 0.95 is 2.4e-7 off: the entry points take doubles and round once, as the tensor operations of torch do, so
+    the moments agree with the oracle to an fp32 rounding or two element by element."""
+    n = 5000
+    p_cpu, m_cpu, v_cpu = make((n,), 5, 0.02), torch.zeros(n), torch.zeros(n)
+    p, m, v = p_cpu.to(DEV), m_cpu.to(DEV), v_cpu.to(DEV)
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    for t in (1, 2, 3):
+        g = make((n,), 50 + t)
+        O.adamw_step(p_cpu, g, m_cpu, v_cpu, t, **kw)
+        F.adamw_step(p, g.to(DEV), m, v, t, **kw)
+        # the same operations in the same order as torch's single-tensor path, each rounded once; torch's CPU
+        # kernels fuse some multiply-adds depending on the host's vector ISA, so the last bit may differ
+        assert float(((v.cpu() - v_cpu).abs() / v_cpu.abs().clamp_min(1e-30)).max()) < 4e-7
+        assert float((m.cpu() - m_cpu).abs().max()) <= 1.2e-7 * float(m_cpu.abs().max())
+        assert float((p.cpu() - p_cpu).abs().max()) <= 1.2e-7 * float(p_cpu.abs().max())
+    # Muon's momentum buffer (fp32 lerp with weight 1 - 0.95)
+    shape = (64, 128)
+    grad, buf = make(shape, 60), make(shape, 61)
+    param = make(shape, 62, 0.02)
+    buf_cpu = buf.clone()
+    O.muon_step(param.clone(), grad, buf_cpu, lr=0.02, weight_decay=0.0, momentum=0.95, nesterov=True)
+    buf_dev = buf.to(DEV)
+    F.muon_step(param.to(DEV), grad.to(DEV), buf_dev, lr=0.02, weight_decay=0.0, momentum=0.95, nesterov=True)
+    assert float((buf_dev.cpu() - buf_cpu).abs().max()) <= 1.2e-7 * float(buf_cpu.abs().max())
+
+
 def test_adamw_unaligned_views_and_errors():
     n = 1001
     base = [torch.zeros(n + 1, device=DEV) for _ in range(3)]

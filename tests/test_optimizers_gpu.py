@@ -89,8 +89,8 @@ def test_fused_adamw_merges_flat_views_into_one_launch_and_matches_torch():
         assert torch.allclose(p.detach().cpu(), r.detach(), rtol=1e-6, atol=1e-8)
         assert torch.allclose(opt.state[p]["exp_avg"].cpu(), opt_ref.state[r]["exp_avg"], rtol=1e-5, atol=1e-10)
         assert float(opt.state[p]["step"]) == 2.0
-    with pytest.raises(NotImplementedError):
-        FusedAdamW(ours, amsgrad=True)
+    with pytest.raises(ValueError, match="Invalid beta"):
+        FusedAdamW(ours, betas=(1.0, 0.9))
 
 
 def build_owner_buffers():

@@ -105,3 +105,25 @@ def test_adamw_step_equals_torch_adamw(wd):
         O.adamw_step(p, g, m, v, t, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=wd)
         assert torch.equal(p, p_ref.detach())
         assert torch.equal(m, opt.state[p_ref]["exp_avg"]) and torch.equal(v, opt.state[p_ref]["exp_avg_sq"])
+
+
+@pytest.mark.parametrize("amsgrad,maximize", [(True, False), (False, True), (True, True)])
+def test_adamw_step_amsgrad_and_maximize_equal_torch_adamw(amsgrad, maximize):
+    """Gradients shrink after the first step, so the running maximum of the second moment differs from the moment
+    itself and a wrong (or missing) maximum changes the result."""
+    p0 = make((1000,), 3, 0.02)
+    grads = [make((1000,), 40 + i) * scale for i, scale in enumerate((1.0, 0.05, 0.2, 0.01))]
+    p_ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([p_ref], lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, amsgrad=amsgrad, maximize=maximize, foreach=False)
+    p, m, v = p0.clone(), torch.zeros(1000), torch.zeros(1000)
+    vmax = torch.zeros(1000) if amsgrad else None
+    for t, g in enumerate(grads, start=1):
+        p_ref.grad = g.clone()
+        opt.step()
+        O.adamw_step(p, g, m, v, t, lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, max_exp_avg_sq=vmax, maximize=maximize)
+        assert torch.equal(p, p_ref.detach())
+        assert torch.equal(m, opt.state[p_ref]["exp_avg"]) and torch.equal(v, opt.state[p_ref]["exp_avg_sq"])
+        if amsgrad:
+            assert torch.equal(vmax, opt.state[p_ref]["max_exp_avg_sq"])
+    if amsgrad:
+        assert not torch.equal(vmax, v)
