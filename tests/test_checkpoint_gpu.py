@@ -621,13 +621,16 @@ def test_dcp_owner_layout_with_mixed_optimizer_into_another_world(tmp_path):
     whole_state = {n: whole_optimizer.state[p] for n, p in whole.named_parameters()}
     whole_params = {n: p.detach().clone() for n, p in whole.named_parameters()}
 
-    source = world(3, [0, 2, 0, 0, 1, 1])  # rank 0 runs AdamW only, rank 2 Muon only, rank 1 both
+    source = world(4, [0, 2, 0, 0, 1, 1])  # rank 0 runs AdamW only, rank 2 Muon only, rank 1 both, rank 3 owns nothing
     for model, optimizer in source:
-        wide_step(model, optimizer)
+        if optimizer is not None:
+            wide_step(model, optimizer)
+    assert source[3][1] is None and source[3][0]._matrix_fsdp_param_group.flat_buffer.local_numel == 0
     save_matrix_dcp_simulated_world([m for m, _ in source], tmp_path, optimizers=[o for _, o in source])
     assert names == ["scale", "up.weight", "up.bias", "norm.weight", "norm.bias", "down.weight"]
     saved = global_metadata(tmp_path)["ranks"]
     assert [set(saved[r]["optimizer"]["components"]) for r in range(3)] == [{"adamw"}, {"muon", "adamw"}, {"muon"}]
+    assert "optimizer" not in saved[3] and saved[3]["param_groups"][0]["shard_sizes"][3] == 0
 
     for rank, (model, optimizer) in enumerate(world(2, [1, 1, 1, 0, 0, 0], seed=5)):
         load_matrix_dcp(model, tmp_path, optimizer=optimizer, allow_reshard=True)
