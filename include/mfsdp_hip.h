@@ -35,6 +35,7 @@ extern "C" {
 /* dtype codes used by the cast / optimizer entry points */
 #define MFSDP_F32 0
 #define MFSDP_BF16 1
+#define MFSDP_F16 2 /* mfsdp_accumulate only */
 
 /* conversion a segment program applies while copying */
 #define MFSDP_CONVERT_NONE 0         /* raw element move, any elem_bytes */
@@ -152,6 +153,14 @@ void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll);
  * _maybe_to_local_dtype (matrix_fsdp/runtime/flat_buffer.py:1186-1206).
  */
 int mfsdp_cast(const void* src, void* dst, int64_t numel, int convert, void* stream);
+
+/*
+ * dst += src over `numel` contiguous elements of one dtype (MFSDP_F32, MFSDP_BF16
+ * or MFSDP_F16; 16-bit formats add in fp32 and round once): a backward that finds
+ * the previous one's reduced gradient shard still in place adds to it,
+ * MatrixFlatBuffer.accumulate_local_grad_shard (matrix_fsdp/runtime/flat_buffer.py:886-900).
+ */
+int mfsdp_accumulate(void* dst, const void* src, int64_t numel, int dtype, void* stream);
 
 /* ------------------------------------------------------------------ Muon */
 

@@ -20,6 +20,7 @@ CONVERT_F16_TO_F32 = 3
 CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
+DT_F16 = 2  # mfsdp_accumulate only
 ABI_VERSION = 1
 
 
@@ -69,6 +70,7 @@ SIGNATURES = {
          c_float, c_float, c_float, c_int, c_float, c_double, c_void_p, c_int64, c_void_p],
     ),
     "mfsdp_set_muon_tuning": (None, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "mfsdp_accumulate": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mfsdp_adamw_step": (
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_double, c_double, c_double, c_double, c_double, c_void_p],

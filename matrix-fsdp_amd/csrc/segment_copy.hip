@@ -714,3 +714,71 @@ extern "C" int mfsdp_cast(const void* src, void* dst, int64_t numel, int convert
   return linear_dispatch(static_cast<const char*>(src), static_cast<char*>(dst), numel, widen ? 2 : 4, widen ? 4 : 2,
                          g_tuning.convert_group, as_stream(stream), is_half_conversion(convert));
 }
+
+// ---- accumulate: dst += src --------------------------------------------------------------------------------------
+
+namespace {
+
+// FMT 0: fp32, 1: bf16, 2: fp16.  16-bit formats add in fp32 and round to nearest even once, as Tensor.add_ does.
+template <int FMT>
+__device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b) {
+  if constexpr (FMT == 0) {
+    return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
+  } else if constexpr (FMT == 1) {
+    const float lo = __uint_as_float(a << 16) + __uint_as_float(b << 16);
+    const float hi = __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u);
+    return f32_bits_to_bf16_bits(__float_as_uint(lo)) | (f32_bits_to_bf16_bits(__float_as_uint(hi)) << 16);
+  } else {
+    const float lo = __uint_as_float(f16_bits_to_f32_bits(a & 0xffffu)) + __uint_as_float(f16_bits_to_f32_bits(b & 0xffffu));
+    const float hi = __uint_as_float(f16_bits_to_f32_bits(a >> 16)) + __uint_as_float(f16_bits_to_f32_bits(b >> 16));
+    return f32_bits_to_f16_bits(__float_as_uint(lo)) | (f32_bits_to_f16_bits(__float_as_uint(hi)) << 16);
+  }
+}
+
+// n_vec 16-byte groups, then `tail` single elements starting at element `tail_first`
+template <int FMT>
+__global__ void __launch_bounds__(kBlockThreads)
+accumulate_kernel(char* __restrict__ dst, const char* __restrict__ src, int64_t n_vec, int64_t tail_first, int64_t tail) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+  for (int64_t g = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; g < n_vec; g += stride) {
+    const Words<16> b = load_bytes<16, true>(src + g * 16);
+    Words<16> a = load_bytes<16, false>(dst + g * 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a.w[i] = add_word<FMT>(a.w[i], b.w[i]);
+    store_bytes<16, false>(dst + g * 16, a);
+  }
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < tail; i += stride) {
+    const int64_t e = tail_first + i;
+    if constexpr (FMT == 0) {
+      reinterpret_cast<float*>(dst)[e] += reinterpret_cast<const float*>(src)[e];
+    } else {
+      uint16_t* d = reinterpret_cast<uint16_t*>(dst) + e;
+      *d = static_cast<uint16_t>(add_word<FMT>(*d, reinterpret_cast<const uint16_t*>(src)[e]));
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int mfsdp_accumulate(void* dst, const void* src, int64_t numel, int dtype, void* stream) {
+  if (numel < 0) return fail(MFSDP_ERR_INVALID, "numel must be non-negative");
+  if (dtype != MFSDP_F32 && dtype != MFSDP_BF16 && dtype != MFSDP_F16) return fail(MFSDP_ERR_INVALID, "dtype must be f32, bf16 or f16");
+  if (numel == 0) return MFSDP_OK;
+  if (dst == nullptr || src == nullptr) return fail(MFSDP_ERR_INVALID, "dst or src is null");
+  const int elem = dtype == MFSDP_F32 ? 4 : 2;
+  const bool aligned = (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16 == 0;
+  const int64_t per_vec = 16 / elem;
+  const int64_t n_vec = aligned ? numel / per_vec : 0;
+  const int64_t tail_first = n_vec * per_vec, tail = numel - tail_first;
+  const int64_t work = std::max(n_vec, tail);
+  const int64_t want = (work + kBlockThreads - 1) / kBlockThreads;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.linear_blocks_per_cu);
+  const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, cap))));
+  char* d = static_cast<char*>(dst);
+  const char* s = static_cast<const char*>(src);
+  if (dtype == MFSDP_F32) hipLaunchKernelGGL((accumulate_kernel<0>), grid, dim3(kBlockThreads), 0, as_stream(stream), d, s, n_vec, tail_first, tail);
+  else if (dtype == MFSDP_BF16) hipLaunchKernelGGL((accumulate_kernel<1>), grid, dim3(kBlockThreads), 0, as_stream(stream), d, s, n_vec, tail_first, tail);
+  else hipLaunchKernelGGL((accumulate_kernel<2>), grid, dim3(kBlockThreads), 0, as_stream(stream), d, s, n_vec, tail_first, tail);
+  MFSDP_CHECK_LAUNCH("accumulate_kernel");
+  return MFSDP_OK;
+}

@@ -145,6 +145,28 @@ def copy_range(input_tensor: torch.Tensor, output_tensor: torch.Tensor, input_of
         )
 
 
+_ACCUMULATE_DTYPES = {torch.float32: _lib.DT_F32, torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16}
+
+
+def accumulate(destination: torch.Tensor, source: torch.Tensor) -> torch.Tensor:
+    """``destination += source`` (``mfsdp_accumulate``) on the current stream:
+    float32, bfloat16 or float16, both contiguous, same dtype and size."""
+    if not (destination.is_cuda and source.is_cuda) or destination.device != source.device:
+        raise RuntimeError("destination and source must be CUDA tensors on one device")
+    if not (destination.is_contiguous() and source.is_contiguous()):
+        raise RuntimeError("destination and source must be contiguous")
+    if destination.dtype != source.dtype or destination.dtype not in _ACCUMULATE_DTYPES:
+        raise RuntimeError(f"accumulate adds float32, bfloat16 or float16 tensors of one dtype, got {destination.dtype} += {source.dtype}")
+    if destination.numel() != source.numel():
+        raise RuntimeError(f"destination has {destination.numel()} elements, source has {source.numel()}")
+    stream = torch.cuda.current_stream(destination.device).cuda_stream
+    with torch.cuda.device(destination.device):
+        _lib.check(
+            _lib.lib().mfsdp_accumulate(destination.data_ptr(), source.data_ptr(), destination.numel(), _ACCUMULATE_DTYPES[destination.dtype], stream)
+        )
+    return destination
+
+
 _CAST_CODES = {
     (torch.bfloat16, torch.float32): _lib.CONVERT_BF16_TO_F32,
     (torch.float32, torch.bfloat16): _lib.CONVERT_F32_TO_BF16,

@@ -446,11 +446,13 @@ class MatrixFlatBuffer:
             self._programs[key] = program
         return program.run(grads, packed_rank_chunks)
 
-    def reduce_grad_bucket_to_local_shard(self, bucket: MatrixGradBucket, *, backend: CopyInBackend = "auto") -> torch.Tensor:
+    def reduce_grad_bucket_to_local_shard(self, bucket: MatrixGradBucket, *, backend: CopyInBackend = "auto", accumulate: bool = False) -> torch.Tensor:
         """Copy-in, then this rank's chunk of the workspace as the local grad
         shard in the local dtype.  Without a process group the reduce-scatter
         is the identity on the rank's chunk (runtime/collectives.py:939-946);
-        grads are therefore not divided by the world size."""
+        grads are therefore not divided by the world size.  ``accumulate`` adds
+        the result to the shard a previous backward left
+        (flat_buffer.py:886-900) instead of replacing it."""
         reduce_dtype = self.reduce_dtype or (bucket.param_grads[0].grad.dtype if bucket.param_grads else self.local_shard.dtype)
         compact = self.is_whole_param_owner_layout() and backend == "auto"
         if bucket.packed_input is not None:
@@ -464,8 +466,43 @@ class MatrixFlatBuffer:
         chunk = torch.empty(self.shard_sizes[self.rank], dtype=packed.dtype, device=self.device)
         offset = self.plan.rank_packed_offset(self.rank) if compact else self.rank * self.layout.max_shard_size
         native.copy_range(packed, chunk, offset)
-        self.local_grad_shard = self._maybe_to_local_dtype(chunk)
+        reduced = self._maybe_to_local_dtype(chunk)
+        if accumulate and self.local_grad_shard is not None:
+            self.accumulate_local_grad_shard(reduced)
+        else:
+            self.local_grad_shard = reduced
         return self.local_grad_shard
+
+    def accumulate_local_grad_shard(self, local_grad_shard: torch.Tensor) -> bool:
+        """Adds a freshly reduced shard to the one already held; returns
+        whether there was one (flat_buffer.py:886-900)."""
+        existing = self.local_grad_shard
+        if existing is None:
+            self.local_grad_shard = local_grad_shard.reshape(-1)
+            return False
+        if existing.numel() != local_grad_shard.numel():
+            raise RuntimeError(f"Accumulated local grad shard has {existing.numel()} elements, new local grad shard has {local_grad_shard.numel()}.")
+        if existing.dtype != local_grad_shard.dtype:
+            local_grad_shard = native.cast(local_grad_shard.contiguous(), existing.dtype)
+        if existing.numel():
+            native.accumulate(existing, local_grad_shard.reshape(-1).contiguous())
+        return True
+
+    def local_grads_are_live(self) -> bool:
+        """Whether some local parameter's ``.grad`` still is a view of the local
+        grad shard (``zero_grad`` has not dropped them)."""
+        if self.local_grad_shard is None:
+            return False
+        storage = self.local_grad_shard.untyped_storage().data_ptr()
+        return any(
+            mp.param.grad is not None and mp.param.grad.untyped_storage().data_ptr() == storage
+            for mp in self.managed_params
+        )
+
+    def detach_param_grads(self) -> None:
+        """``param.grad = None`` everywhere; the shard itself stays with the buffer."""
+        for mp in self.managed_params:
+            mp.param.grad = None
 
     def use_local_grad_shard(self, local_grad_shard: torch.Tensor | None = None) -> None:
         """``param.grad`` -> views of the reduced local grad shard, which a

@@ -124,6 +124,7 @@ class MatrixFSDPParamGroup:
         self._expected_param_ids: set[int] = set()
         self._backward_callback_queued = False
         self._finalized_after_backward = True
+        self._grads_stashed = False
         self.init()
 
     # ------------------------------------------------------------------ set-up
@@ -189,6 +190,7 @@ class MatrixFSDPParamGroup:
         self._seen_param_ids.clear()
         self._backward_callback_queued = False
         self._finalized_after_backward = True
+        self._grads_stashed = False
 
     def remove_hooks(self) -> None:
         for handle in self._handles:
@@ -255,10 +257,25 @@ class MatrixFSDPParamGroup:
         return output
 
     # ------------------------------------------------------------------ backward
+    def _stash_local_grads(self) -> None:
+        """Before autograd writes this backward's full gradients: the reduced
+        shard of an earlier backward stays with the flat buffer if the
+        parameters still point at it (this backward then adds to it, as
+        ``.grad`` accumulates everywhere in torch) and is dropped if
+        ``zero_grad`` has cleared them; either way ``param.grad`` is emptied, a
+        local-shard view cannot receive a full gradient."""
+        fb = self.flat_buffer
+        if fb.local_grad_shard is not None and not fb.local_grads_are_live():
+            fb.clear_local_grad_shard()
+        fb.detach_param_grads()
+
     def _pre_backward(self, grad: torch.Tensor) -> torch.Tensor:
         if not self._backward_callback_queued:
             self._backward_callback_queued = True
             Variable._execution_engine.queue_callback(self._post_backward_callback)
+        if not self._grads_stashed and not self._finalized_after_backward:
+            self._grads_stashed = True
+            self._stash_local_grads()
         if self.lifecycle_state != FSDPLifecycleState.UNSHARDED and not self._finalized_after_backward:
             self._record("pre_backward")
             self.unshard("pre_backward")
@@ -295,12 +312,18 @@ class MatrixFSDPParamGroup:
                 by_fqn.update({mp.fqn: BucketParamGrad(mp, z) for mp, z in zeros})
                 ordered = tuple(by_fqn[mp.fqn] for mp in self.managed_params)
                 bucket = MatrixGradBucket(ordered, bucket.total_numel, bucket.shard_sizes, bucket.rank_segments)
-            fb.reduce_grad_bucket_to_local_shard(bucket)
+            accumulated = fb.local_grad_shard is not None
+            fb.reduce_grad_bucket_to_local_shard(bucket, accumulate=True)
             fb.use_local_shards()
             fb.use_local_grad_shard()
+            if accumulated:
+                self._record("accumulate_local_grad_shard")
         else:
             fb.use_local_shards()
+            if fb.local_grad_shard is not None:
+                fb.use_local_grad_shard()  # nothing new: the stashed shard goes back to the parameters
         self.lifecycle_state = FSDPLifecycleState.SHARDED
         self._finalized_after_backward = True
+        self._grads_stashed = False
         self._seen_param_ids.clear()
         self._record("finalize_backward")

@@ -242,6 +242,24 @@ def test_fp16_casts_match_tensor_to():
         assert torch.equal(gathered.cpu().view(torch.int16), O.pack_to_padded(full, plan).to(torch.float16).view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_accumulate_matches_tensor_add(dtype):
+    gen = torch.Generator().manual_seed(12)
+    for n, shift in ((1 << 16, 0), (4099, 0), (4099, 1), (13, 3), (1, 0), (0, 0)):
+        a = (torch.randn(n + shift, generator=gen) * 3).to(dtype)
+        b = (torch.randn(n + shift, generator=gen) * 3).to(dtype)
+        have = a.to(DEV)[shift:]
+        have = have if shift == 0 else have  # a view that starts off the 16-byte grid when shift > 0
+        out = native.accumulate(have, b.to(DEV)[shift:])
+        assert out is have
+        want = a[shift:].clone().add_(b[shift:])
+        assert torch.equal(have.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32), want.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    with pytest.raises(RuntimeError, match="one dtype"):
+        native.accumulate(torch.zeros(4, device=DEV), torch.zeros(4, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="elements"):
+        native.accumulate(torch.zeros(4, device=DEV), torch.zeros(5, device=DEV))
+
+
 def test_random_layouts_every_width():
     rng = random.Random(1)
     for trial in range(40):

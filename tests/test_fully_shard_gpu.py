@@ -199,6 +199,41 @@ def test_mixed_precision_low_precision_compute_fp32_master(low):
         assert rel(have[name], want[name]) < 2e-6, name
 
 
+@pytest.mark.parametrize("world, rank", [(1, 0), (4, 1)])
+def test_gradients_accumulate_over_backwards_until_zero_grad(world, rank):
+    """Micro-batches: every backward reduces its gradients into the local shard and adds them to what the
+    previous one left, ``zero_grad`` (dropping or zeroing the grads) starts over.  The twin accumulates full
+    gradients in ``.grad`` the ordinary way; the rank's shard of them is compared bit for bit (fp32 adds of the
+    same numbers in the same order)."""
+    model, twin = make_pair(seed=5)
+    shard_all(model, world_size=world, rank=rank, planner=fsdp2_chunk_plan)
+    units = [m._matrix_fsdp_param_group for m in [*model.blocks, model]]
+    opt = configure_optimizer(model, "adamw", lr=1e-3)
+
+    def twin_local_grads(unit):
+        full = torch.cat([dict(twin.named_parameters())[prefix + mp.fqn].grad.reshape(-1) for prefix, u in prefixed if u is unit for mp in u.managed_params])
+        return torch.cat([full[s.global_start : s.global_end] for s in unit.flat_buffer.local_segments])
+
+    prefixed = [(f"blocks.{i}.", u) for i, u in enumerate(units[:-1])] + [("", units[-1])]
+    data = batches(4, seed=9)
+    for round_, zero in enumerate(("none", "zeros")):
+        for micro, (x, y) in enumerate(data[2 * round_ : 2 * round_ + 2]):
+            torch.nn.functional.mse_loss(model(x), y).backward()
+            torch.nn.functional.mse_loss(twin(x), y).backward()
+            for unit in units:
+                fb = unit.flat_buffer
+                assert torch.equal(fb.local_grad_shard, twin_local_grads(unit)), (round_, micro)
+                assert all(v.managed_param.param.grad.data_ptr() == fb.local_grad_shard.data_ptr() + v.shard_start * 4 for v in fb.local_param_views)
+                assert ("accumulate_local_grad_shard" in unit.events[-3:]) == (micro == 1)
+        # no step: the parameters of the two models stay identical, so the gradients can be compared bit for bit
+        opt.zero_grad(set_to_none=(zero == "none"))
+        twin.zero_grad(set_to_none=(zero == "none"))
+        if zero == "none":
+            assert all(p.grad is None for p in model.parameters())
+        else:
+            assert all(float(u.flat_buffer.local_grad_shard.abs().sum()) == 0.0 for u in units)
+
+
 def test_simulated_world_of_four_updates_only_the_rank_shard():
     """Rank 1 of a simulated world of 4 (per-parameter chunks): parameters are packed, gathered and unpacked
     through the segment programs every step, and the optimizer sees quarter-parameter views.  The twin trains
