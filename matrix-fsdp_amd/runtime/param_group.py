@@ -134,6 +134,10 @@ class MatrixFSDPParamGroup:
         self.managed_params = list(
             managed_params_from_module(self.module, shard_hints=self.shard_hints, ignored_params=self.ignored_params | taken)
         )
+        # frozen parameters would be handed zero gradients by the reduced shard and then decayed by the optimizer;
+        # the reference refuses them (fsdp_unit.py:1694-1703): pass them as ignored_params instead
+        if any(not mp.param.requires_grad for mp in self.managed_params):
+            raise NotImplementedError("MatrixFSDP V0 expects all managed parameters to require grad.")
         self.module._matrix_fsdp_param_group = self  # type: ignore[attr-defined]
         if not self.managed_params:
             return
