@@ -124,7 +124,7 @@ class MatrixFSDPParamGroup:
         self._expected_param_ids: set[int] = set()
         self._backward_callback_queued = False
         self._finalized_after_backward = True
-        self._grads_stashed = False
+        self._in_backward = False
         self.init()
 
     # ------------------------------------------------------------------ set-up
@@ -194,7 +194,7 @@ class MatrixFSDPParamGroup:
         self._seen_param_ids.clear()
         self._backward_callback_queued = False
         self._finalized_after_backward = True
-        self._grads_stashed = False
+        self._in_backward = False
 
     def remove_hooks(self) -> None:
         for handle in self._handles:
@@ -231,6 +231,14 @@ class MatrixFSDPParamGroup:
     def _pre_forward(self, module, args, kwargs):
         if self.flat_buffer is None:
             return args, kwargs
+        if self._in_backward:
+            # activation checkpointing re-runs the forward in the middle of this unit's backward: the parameters
+            # are (or become) full again and the bookkeeping of the backward in flight is left alone
+            self.unshard("recompute")
+            if self.cast_forward_inputs and self.param_dtype is not None:
+                args = _floating_tensors_to(args, self.param_dtype)
+                kwargs = _floating_tensors_to(kwargs, self.param_dtype)
+            return args, kwargs
         if not self._finalized_after_backward and self.lifecycle_state == FSDPLifecycleState.FORWARD_RESHARDED:
             raise RuntimeError(
                 "reshard_after_forward=True does not support running another forward before the previous forward has entered backward."
@@ -246,6 +254,8 @@ class MatrixFSDPParamGroup:
     def _post_forward(self, module, args, kwargs, output):
         if self.flat_buffer is None:
             return output
+        if self._in_backward:  # a recomputed forward: no reshard, no new backward hooks
+            return output if self.output_dtype is None else _floating_tensors_to(output, self.output_dtype)
         grad_enabled = torch.is_grad_enabled()
         outputs_with_grad = list(_tensors_requiring_grad(output)) if grad_enabled else []
         if outputs_with_grad:
@@ -277,8 +287,8 @@ class MatrixFSDPParamGroup:
         if not self._backward_callback_queued:
             self._backward_callback_queued = True
             Variable._execution_engine.queue_callback(self._post_backward_callback)
-        if not self._grads_stashed and not self._finalized_after_backward:
-            self._grads_stashed = True
+        if not self._in_backward and not self._finalized_after_backward:
+            self._in_backward = True  # until finalize_backward
             self._stash_local_grads()
         if self.lifecycle_state != FSDPLifecycleState.UNSHARDED and not self._finalized_after_backward:
             self._record("pre_backward")
@@ -328,6 +338,6 @@ class MatrixFSDPParamGroup:
                 fb.use_local_grad_shard()  # nothing new: the stashed shard goes back to the parameters
         self.lifecycle_state = FSDPLifecycleState.SHARDED
         self._finalized_after_backward = True
-        self._grads_stashed = False
+        self._in_backward = False
         self._seen_param_ids.clear()
         self._record("finalize_backward")

@@ -234,6 +234,75 @@ def test_gradients_accumulate_over_backwards_until_zero_grad(world, rank):
             assert all(float(u.flat_buffer.local_grad_shard.abs().sum()) == 0.0 for u in units)
 
 
+class CheckpointedNet(Net):
+    """Every block runs under activation checkpointing: its forward is re-run in the middle of the backward."""
+
+    use_reentrant = False
+
+    def forward(self, x):
+        from torch.utils.checkpoint import checkpoint
+
+        for block in self.blocks:
+            x = checkpoint(block, x, use_reentrant=self.use_reentrant)
+        return self.head(x)
+
+
+@pytest.mark.parametrize("use_reentrant", [False, True])
+@pytest.mark.parametrize("reshard_after_forward", [True, False])
+@pytest.mark.parametrize("world, rank", [(1, 0), (4, 2)])
+def test_activation_checkpointing_recomputes_inside_the_backward(use_reentrant, reshard_after_forward, world, rank):
+    torch.manual_seed(6)
+    model = CheckpointedNet().to(DEV)
+    model.use_reentrant = use_reentrant
+    twin = Net().to(DEV)
+    twin.load_state_dict(model.state_dict())
+    shard_all(model, world_size=world, rank=rank, planner=fsdp2_chunk_plan, reshard_after_forward=reshard_after_forward)
+    units = [m._matrix_fsdp_param_group for m in [*model.blocks, model]]
+    names = [(f"blocks.{i}.", u) for i, u in enumerate(units[:-1])] + [("", units[-1])]
+    for x, y in batches(2, seed=11):
+        for unit in units:
+            unit.events.clear()
+        x = x.requires_grad_(use_reentrant)  # the reentrant form needs an input that requires grad
+        torch.nn.functional.mse_loss(model(x), y).backward()
+        torch.nn.functional.mse_loss(twin(x.detach()), y).backward()
+        for prefix, unit in names:
+            assert unit.lifecycle_state == FSDPLifecycleState.SHARDED and not unit._in_backward
+            fb = unit.flat_buffer
+            full = torch.cat([dict(twin.named_parameters())[prefix + mp.fqn].grad.reshape(-1) for mp in unit.managed_params])
+            want = torch.cat([full[s.global_start : s.global_end] for s in fb.local_segments])
+            assert torch.equal(fb.local_grad_shard, want), prefix
+        if not use_reentrant:  # the re-run forward neither reshards nor counts as a new forward
+            assert units[0].events.count("pre_forward") == 1
+            assert units[0].events.count("reshard:post_forward") == int(reshard_after_forward)
+        for p in [*model.parameters(), *twin.parameters()]:
+            p.grad = None
+
+
+def test_a_unit_called_twice_in_one_forward_and_an_unused_unit():
+    """Weight sharing in time: the same block applied twice before one backward (``reshard_after_forward=False``,
+    with resharding the second forward is refused), and a unit that takes no part in the step at all."""
+    model, twin = make_pair(seed=8)
+    shard_all(model, reshard_after_forward=False)
+    units = [m._matrix_fsdp_param_group for m in [*model.blocks, model]]
+    (x, y), = batches(1, seed=12)
+
+    def twice(net, x):
+        return net.head(net.blocks[0](net.blocks[0](x)))  # blocks[1] unused; the root's own forward is bypassed too
+
+    torch.nn.functional.mse_loss(twice(model, x), y).backward()
+    torch.nn.functional.mse_loss(twice(twin, x), y).backward()
+    assert units[0].lifecycle_state == FSDPLifecycleState.SHARDED
+    for (name, p), q in zip(model.blocks[0].named_parameters(), twin.blocks[0].parameters()):
+        assert torch.equal(p.grad, q.grad), name
+    assert all(p.grad is None for p in model.blocks[1].parameters())  # nothing reduced, nothing to step
+    assert units[1].flat_buffer.local_grad_shard is None
+
+    strict, _ = make_pair(seed=8)
+    fully_shard(strict.blocks[0])
+    with pytest.raises(RuntimeError, match="another forward"):
+        strict.blocks[0](strict.blocks[0](x))
+
+
 def test_simulated_world_of_four_updates_only_the_rank_shard():
     """Rank 1 of a simulated world of 4 (per-parameter chunks): parameters are packed, gathered and unpacked
     through the segment programs every step, and the optimizer sees quarter-parameter views.  The twin trains
