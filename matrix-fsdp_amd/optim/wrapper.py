@@ -158,7 +158,9 @@ class MixedMuonAdamWOptimizer:
         muon_adjust_lr_fn: str | None = DEFAULT_MUON_ADJUST_LR_FN,
         flat_adamw_state: bool = False,
         flat_buffers: Iterable | None = None,
+        fsdp_param_groups: Iterable | None = None,
     ) -> None:
+        self.fsdp_param_groups = list(fsdp_param_groups or ())
         self.muon_params = tuple(p for p in muon_params if p.numel() > 0)
         self.adamw_params = tuple(p for p in adamw_params if p.numel() > 0)
         self.group_summaries = tuple(group_summaries)
@@ -212,6 +214,7 @@ class MixedMuonAdamWOptimizer:
     def step(self, closure=None):
         if closure is not None:
             raise NotImplementedError("MixedMuonAdamWOptimizer does not support closures.")
+        prepare_units_for_step(self.fsdp_param_groups)
         if self.flat_adamw_state and self.adamw is not None and self.flat_buffers:
             initialize_flat_adamw_state(self.adamw, self.flat_buffers)
         result = None
@@ -255,8 +258,31 @@ class MixedMuonAdamWOptimizer:
         }
 
 
+def units_of(module_or_units) -> list:
+    """The lifecycle units behind ``module_or_units`` (none for bare flat buffers)."""
+    if isinstance(module_or_units, nn.Module) or hasattr(module_or_units, "finalize_backward"):
+        return collect_param_groups(module_or_units)
+    if hasattr(module_or_units, "local_param_views"):
+        return []
+    return [item for item in module_or_units if hasattr(item, "finalize_backward")]
+
+
+def prepare_units_for_step(units, operation: str = "optimizer.step") -> None:
+    for unit in units:
+        unit.prepare_for_optimizer_step(operation)
+
+
+def _manage_lifecycle(optimizer: torch.optim.Optimizer, units: list) -> None:
+    """``optimizer.step()`` first finishes pending backwards and insists on
+    sharded parameters, as the reference's prepared optimizers do
+    (matrix_fsdp/optim/wrapper.py:227-241, 957-977)."""
+    if units:
+        optimizer.register_step_pre_hook(lambda opt, args, kwargs: prepare_units_for_step(units))
+
+
 def make_mixed_muon_adamw_optimizer(module_or_units, *, default_matrix_optimizer: str = "muon", default_other_optimizer: str = "adamw", **optimizer_kwargs: Any) -> MixedMuonAdamWOptimizer:
     flat_buffers = collect_flat_buffers(module_or_units)
+    optimizer_kwargs.setdefault("fsdp_param_groups", units_of(module_or_units))
     classified = classify_matrix_optimizer_params(
         flat_buffers, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer
     )
@@ -299,11 +325,16 @@ def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig 
         )
     params = _local_params(module_or_units)
     if kind == "adamw":
-        return FusedAdamW(params, **optimizer_kwargs)
-    if kind == "sgd":
-        return torch.optim.SGD(params, **optimizer_kwargs)
-    if kind == "muon":
-        return Muon(params, **optimizer_kwargs)
+        built = FusedAdamW(params, **optimizer_kwargs)
+    elif kind == "sgd":
+        built = torch.optim.SGD(params, **optimizer_kwargs)
+    elif kind == "muon":
+        built = Muon(params, **optimizer_kwargs)
+    else:
+        built = None
+    if built is not None:
+        _manage_lifecycle(built, units_of(module_or_units))
+        return built
     raise ValueError(f"optimizer must be one of 'adamw', 'sgd', 'muon', or 'mixed_muon_adamw', got {kind!r}.")
 
 
@@ -357,8 +388,7 @@ class MatrixFSDPOptimizer:
     def step(self, closure=None):
         if closure is not None:
             raise NotImplementedError("MatrixFSDPOptimizer V0 does not support optimizer closures.")
-        for unit in self._fsdp_param_groups:
-            unit.finalize_backward()  # a no-op once the autograd pass has finalised the unit
+        prepare_units_for_step(self._fsdp_param_groups, "MatrixFSDPOptimizer.step()")
         if self.flat_adamw_state and isinstance(self.optimizer, torch.optim.Optimizer):
             initialize_flat_adamw_state(self.optimizer, collect_flat_buffers(self._fsdp_param_groups))
         result = self.optimizer.step()

@@ -188,6 +188,27 @@ class MatrixFSDPParamGroup:
             "cast_forward_inputs": bool(self.cast_forward_inputs),
         }
 
+    def assert_optimizer_ready(self, operation: str = "optimizer.step") -> None:
+        """An optimizer may only touch the parameters while they are views of
+        the local shard (matrix_fsdp/runtime/fsdp_unit.py:905-915)."""
+        if self.flat_buffer is not None and self.lifecycle_state != FSDPLifecycleState.SHARDED:
+            raise RuntimeError(
+                f"{operation} expects MatrixFSDP parameters to be sharded, "
+                f"but found lifecycle state {self.lifecycle_state.value}."
+            )
+
+    def prepare_for_optimizer_step(self, operation: str = "optimizer.step") -> None:
+        """Finishes a backward that has not been finalised yet, then checks
+        that the unit is sharded.  A forward whose backward has not started
+        leaves the unit forward-resharded: stepping there is refused."""
+        if self.flat_buffer is None:
+            return
+        if self.lifecycle_state == FSDPLifecycleState.FORWARD_RESHARDED:
+            raise RuntimeError(f"{operation} cannot run on a forward-resharded MatrixFSDP unit: run backward first.")
+        if self._in_backward:
+            self.finalize_backward()
+        self.assert_optimizer_ready(operation)
+
     def reset_after_load(self) -> None:
         """A checkpoint load leaves the unit sharded with no backward pending."""
         self.lifecycle_state = FSDPLifecycleState.SHARDED

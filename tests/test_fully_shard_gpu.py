@@ -377,13 +377,27 @@ def test_lifecycle_rules():
     with torch.no_grad():
         model(x)
     assert unit.lifecycle_state == FSDPLifecycleState.SHARDED and unit.flat_buffer.param_data_alias_local_shard()
+    opt = configure_optimizer(model, "adamw", lr=1e-3)
+    mixed = configure_optimizer(model, "mixed_muon_adamw", lr=1e-3)
     out = model(x)
     assert unit.lifecycle_state == FSDPLifecycleState.FORWARD_RESHARDED
     with pytest.raises(RuntimeError, match="another forward"):
         model(x)
+    for optimizer in (opt, mixed):  # between forward and backward there is nothing to step
+        with pytest.raises(RuntimeError, match="forward-resharded"):
+            optimizer.step()
     out.sum().backward()
     assert unit.lifecycle_state == FSDPLifecycleState.SHARDED
     assert "unshard:pre_backward" in unit.events and unit.events[-1] == "finalize_backward"
+    unit.unshard()
+    with pytest.raises(RuntimeError, match="expects MatrixFSDP parameters to be sharded"):
+        opt.step()
+    with pytest.raises(RuntimeError, match="expects MatrixFSDP parameters to be sharded"):
+        unit.assert_optimizer_ready("test")
+    unit.reshard()
+    before = unit.flat_buffer.local_shard.clone()
+    opt.step()
+    assert not torch.equal(unit.flat_buffer.local_shard, before)
     with pytest.raises(ValueError, match="already wrapped"):
         fully_shard(model)
     with pytest.raises(ValueError, match="floating-point"):
