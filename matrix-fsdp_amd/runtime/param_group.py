@@ -77,6 +77,38 @@ def _tensors_requiring_grad(obj) -> Iterable[torch.Tensor]:
             yield from _tensors_requiring_grad(o)
 
 
+class MatrixFSDPNoSync:
+    """``with model.no_sync():`` -- micro-batches whose gradients are to be
+    accumulated before the next optimizer step (matrix_fsdp/runtime/fsdp_unit.py:70-97).
+    On one device the "reduce" of a backward is a local copy-in, so nothing is
+    deferred: every backward adds its reduced shard to the accumulated one, in
+    and out of this context, and the result is what the reference reaches at
+    the first backward outside it.  What the context keeps is the rule that
+    ``optimizer.step()`` may not run inside it."""
+
+    def __init__(self, units: Iterable["MatrixFSDPParamGroup"]) -> None:
+        self.units = list(units)
+
+    def __enter__(self) -> "MatrixFSDPNoSync":
+        for unit in self.units:
+            unit._no_sync_depth += 1
+        return self
+
+    def __exit__(self, *exc) -> None:
+        for unit in self.units:
+            unit._no_sync_depth -= 1
+
+
+def _units_below(module: nn.Module) -> list["MatrixFSDPParamGroup"]:
+    found, seen = [], set()
+    for sub in module.modules():
+        unit = getattr(sub, "_matrix_fsdp_param_group", None)
+        if unit is not None and id(unit) not in seen:
+            seen.add(id(unit))
+            found.append(unit)
+    return found
+
+
 class MatrixFSDPParamGroup:
     def __init__(
         self,
@@ -125,6 +157,7 @@ class MatrixFSDPParamGroup:
         self._backward_callback_queued = False
         self._finalized_after_backward = True
         self._in_backward = False
+        self._no_sync_depth = 0
         self.init()
 
     # ------------------------------------------------------------------ set-up
@@ -139,6 +172,8 @@ class MatrixFSDPParamGroup:
         if any(not mp.param.requires_grad for mp in self.managed_params):
             raise NotImplementedError("MatrixFSDP V0 expects all managed parameters to require grad.")
         self.module._matrix_fsdp_param_group = self  # type: ignore[attr-defined]
+        module = self.module
+        self.module.no_sync = lambda: MatrixFSDPNoSync(_units_below(module))  # type: ignore[attr-defined]
         if not self.managed_params:
             return
         plan = self.planner(self.managed_params, self.world_size)
@@ -188,6 +223,12 @@ class MatrixFSDPParamGroup:
             "cast_forward_inputs": bool(self.cast_forward_inputs),
         }
 
+    def no_sync(self) -> MatrixFSDPNoSync:
+        return MatrixFSDPNoSync([self])
+
+    def is_no_sync_active(self) -> bool:
+        return self._no_sync_depth > 0
+
     def assert_optimizer_ready(self, operation: str = "optimizer.step") -> None:
         """An optimizer may only touch the parameters while they are views of
         the local shard (matrix_fsdp/runtime/fsdp_unit.py:905-915)."""
@@ -201,6 +242,8 @@ class MatrixFSDPParamGroup:
         """Finishes a backward that has not been finalised yet, then checks
         that the unit is sharded.  A forward whose backward has not started
         leaves the unit forward-resharded: stepping there is refused."""
+        if self._no_sync_depth > 0:
+            raise RuntimeError(f"{operation} cannot run inside MatrixFSDP no_sync().")
         if self.flat_buffer is None:
             return
         if self.lifecycle_state == FSDPLifecycleState.FORWARD_RESHARDED:

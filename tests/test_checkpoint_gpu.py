@@ -482,7 +482,7 @@ def test_state_manager_describes_shard_shaped_state():
     states = [s for p, s in optimizer.optimizer.state.items() if p.numel()]
     assert {s["max_exp_avg_sq"].untyped_storage().data_ptr() for s in states} == {flat.max_exp_avg_sq.untyped_storage().data_ptr()}
     for have, want in zip(model.parameters(), twin.parameters()):
-        assert torch.allclose(have.detach(), want.detach(), rtol=0, atol=2e-6 * float(want.abs().max()))
+        assert torch.allclose(have.detach(), want.detach(), rtol=0, atol=2e-6 * float(want.detach().abs().max()))
         assert torch.allclose(optimizer.state[have]["max_exp_avg_sq"], reference.state[want]["max_exp_avg_sq"], rtol=1e-5, atol=1e-10)
 
     # opt-in only

@@ -395,6 +395,11 @@ def test_lifecycle_rules():
     with pytest.raises(RuntimeError, match="expects MatrixFSDP parameters to be sharded"):
         unit.assert_optimizer_ready("test")
     unit.reshard()
+    with model.no_sync():  # covers every unit below the module it is called on
+        assert unit.is_no_sync_active()
+        with pytest.raises(RuntimeError, match="no_sync"):
+            opt.step()
+    assert not unit.is_no_sync_active()
     before = unit.flat_buffer.local_shard.clone()
     opt.step()
     assert not torch.equal(unit.flat_buffer.local_shard, before)
