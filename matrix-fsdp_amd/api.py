@@ -74,6 +74,9 @@ def matrix_fully_shard(
     an owner rank (the other planner families of the reference do not exist
     here)."""
     validate_mixed_precision_policy(mp_policy)
+    if not isinstance(reshard_after_forward, bool):
+        # an int asks for resharding to a smaller world after forward (matrix_fsdp/runtime/fsdp_unit.py:1705-1720)
+        raise NotImplementedError("reshard_after_forward=int requires post-forward subgroup resharding, which does not exist here; pass a bool.")
     if auto_planner_policy is not None:
         if str(auto_planner_policy).lower() != "muon_shard_aware":
             raise ValueError(f"auto_planner_policy={auto_planner_policy!r} is not available; only 'muon_shard_aware' is.")
@@ -173,6 +176,6 @@ def fully_shard(
         planner=planner,
         shard_hints=hints or None,
         ignored_params=ignored_params,
-        reshard_after_forward=True if reshard_after_forward is None else bool(reshard_after_forward),
+        reshard_after_forward=True if reshard_after_forward is None else reshard_after_forward,
         mp_policy=mp_policy,
     )

@@ -242,6 +242,8 @@ def test_fully_shard_host_rules():
         matrix_fully_shard(module, auto_planner_policy="muon_shard_aware", planner=default_planner)
     with pytest.raises(RuntimeError, match="HIP device"):
         matrix_fully_shard(module, wrap_policy=module_type_policy(torch.nn.Linear))
+    with pytest.raises(NotImplementedError, match="subgroup resharding"):
+        fully_shard(module, reshard_after_forward=2)
     frozen = torch.nn.Linear(2, 2)
     frozen.bias.requires_grad_(False)
     with pytest.raises(NotImplementedError, match="require grad"):
