@@ -199,7 +199,8 @@ int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype
 
 /* Kernel selection for experiments (values <= 0 keep the current setting):
  * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
- * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU), a reserved argument (slabs always stream
+ * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU; for the symmetric products also 3, the default:
+ * whichever of the two fills the CUs better for the size at hand), a reserved argument (slabs always stream
  * HBM -> LDS directly), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
  * stagger >= 0 sets the K-walk start offset, in 64-element slabs, between consecutive tiles. */
 void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,

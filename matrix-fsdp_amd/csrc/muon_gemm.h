@@ -35,7 +35,7 @@ constexpr int64_t kGemmPartialsBytes = 64ll << 20;
 
 struct GemmTuning {
   int general_variant = 1;    // 1: 256x256 tile / 8 waves / one workgroup per CU, 2: 128x128 tile / 4 waves / two per CU
-  int symmetric_variant = 2;
+  int symmetric_variant = 3;  // 1, 2 as above; 3: whichever fills the CUs better for the product at hand
   int direct_to_lds = 1;      // reserved (slabs always stream HBM -> LDS directly)
   int split_remainder = 1;    // split the tiles of the last partial round along K
   int max_splits = 16;

@@ -511,7 +511,29 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
       (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
-  const int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
+  int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
+  if (a.symmetric && variant == 3) {
+    // The triangle of a symmetric product rarely tiles the machine evenly.  Compare the two tilings in rounds of
+    // resident workgroups, the last partial round counting 1/splits (plus the partial-tile traffic, which grows with
+    // the splits) when its tiles are split along K: a round of 128x128 tiles (two per CU) takes about 0.6 of a round
+    // of 256x256 tiles.  m = 4096 on 256 CUs: 136 big tiles are one half-empty round (1.0) against 528 small ones in
+    // 1 + 1/16 rounds (0.83); m = 5120: 210 big tiles in one round (1.0) against 820 small ones in two (1.2) --
+    // measured 15 % faster with the big tiles.  Below three quarters of a round of big tiles (m <= 4096 on 256 CUs)
+    // only K-splitting would fill the machine and the small tiles win (m = 3072: 0.89 ms against 1.15 ms for the five
+    // iterations; m = 2048, k = 8192: 0.88 against 0.99).
+    auto rounds = [&](int tile, int per_cu) {
+      const int t = a.M / tile, tiles = t * (t + 1) / 2, slots = device_cu_count() * per_cu;
+      const int rem = tiles % slots;
+      double r = tiles / slots;
+      if (rem != 0) {
+        const int splits = g_tuning.split_remainder ? std::min({slots / rem, a.K / kSlabK, g_tuning.max_splits}) : 1;
+        r += splits > 1 ? 1.0 / splits + 0.02 * splits : 1.0;
+      }
+      return r;
+    };
+    const int big = a.M / 256, big_tiles = big * (big + 1) / 2;
+    variant = (4 * big_tiles >= 3 * device_cu_count() && rounds(256, 1) <= 0.6 * rounds(128, 2)) ? 1 : 2;
+  }
   // Slabs of 32 (three to five deep) were measured too: each slab row is then half a 128-byte line, the vector
   // cache looks every line up twice, and the products run 15-25 % slower than with slabs of 64 two deep.
   if (variant == 2)  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
