@@ -10,13 +10,16 @@ collectives, prefetching, offload or the planner families are not accepted.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from functools import partial
 from typing import Callable, Mapping
 
 import torch
 from torch import nn
+from torch.distributed.tensor import Shard
 
 from .core.layout import ShardPlan
 from .core.managed_param import ManagedParam, ParamShardHint
+from .planning.group_plans import hinted_ordered_group_plan
 from .planning.owner_plans import MuonOwnerPlanner
 from .planning.shard_hint import build_shard_hints
 from .policy.wrap import WrapPolicy
@@ -129,21 +132,34 @@ def _wrap_selected(module: nn.Module, wrap_policy: WrapPolicy, ignored_params, a
     return sum(_wrap_selected(child, wrap_policy, ignored_params, auto_shard_hints, unit_args) for child in module.children())
 
 
+def _leading_dim_shard_hint(fqn: str, param: nn.Parameter) -> ParamShardHint:
+    """``Shard(0)`` as a hint: a matrix may be cut between any two rows, any other
+    tensor between any two slices along its first dimension (matrix_fsdp/api.py:159-167)."""
+    if param.ndim == 0:
+        raise NotImplementedError(f"MatrixFSDP cannot apply Shard(0) to scalar parameter {fqn}.")
+    if param.ndim == 2:
+        return ParamShardHint(split_granularity="row_block", block_shape=(1, int(param.shape[1])))
+    return ParamShardHint(split_granularity="block", block_shape=(int(param.numel() // param.shape[0]),))
+
+
 def fully_shard(
     module: nn.Module,
     *,
     world_size: int = 1,
     rank: int = 0,
     reshard_after_forward: bool | None = None,
-    shard_placement_fn: Callable[[nn.Parameter], ParamShardHint | None] | None = None,
+    shard_placement_fn: Callable[[nn.Parameter], object | None] | None = None,
     mp_policy=_DEFAULT_MP_POLICY,
     ignored_params: set[nn.Parameter] | None = None,
     planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
     optimizer_policy: str | None = None,
 ) -> nn.Module:
     """FSDP2-style spelling (matrix_fsdp/api.py:213-263): ``shard_placement_fn``
-    maps a parameter to a ``ParamShardHint`` (or ``None``); ``reshard_after_forward``
-    defaults to ``True``.  A Muon ``optimizer_policy`` (``"muon"``,
+    maps a parameter to ``torch.distributed.tensor.Shard(0)`` or ``None`` (a
+    ``ParamShardHint`` is accepted as well); parameters placed with ``Shard(0)``
+    may be cut between rows (first-dimension slices) and the unit's flat buffer
+    is then cut rank-contiguously at such boundaries (``hinted_ordered_group_plan``);
+    ``reshard_after_forward`` defaults to ``True``.  A Muon ``optimizer_policy`` (``"muon"``,
     ``"mixed_muon_adamw"``, ...) derives the hints from the module structure
     (``build_shard_hints``) and keeps every parameter whole on an owner rank
     (``MuonOwnerPlanner``; pass one planner object to all units to balance the
@@ -161,14 +177,30 @@ def fully_shard(
             raise ValueError(f"Unknown fully_shard optimizer_policy={optimizer_policy!r}; expected one of {allowed}.")
     if shard_placement_fn is not None:
         ignored = {id(p) for p in ignored_params or ()}
+        placed = False
         for fqn, param in module.named_parameters():
             if id(param) in ignored or getattr(param, "_matrix_fsdp_managed", False):
                 continue
-            hint = shard_placement_fn(param)
-            if hint is not None:
-                if not isinstance(hint, ParamShardHint):
-                    raise TypeError(f"shard_placement_fn must return ParamShardHint or None, got {type(hint).__name__} for {fqn}.")
-                hints[fqn] = hint
+            placement = shard_placement_fn(param)
+            if placement is None:
+                continue
+            if isinstance(placement, ParamShardHint):  # an explicit hint is taken as it is
+                hints[fqn] = placement
+                continue
+            if not isinstance(placement, Shard):
+                raise NotImplementedError(
+                    "MatrixFSDP fully_shard shard_placement_fn currently supports only None or torch.distributed.tensor.Shard placements."
+                )
+            if placement.dim != 0:
+                raise NotImplementedError(
+                    "MatrixFSDP fully_shard shard_placement_fn currently supports only Shard(0). Sharding non-leading tensor "
+                    "dimensions would require non-contiguous local storage segments."
+                )
+            hints[fqn] = _leading_dim_shard_hint(fqn, param)
+            placed = True
+        if placed and planner is None:
+            # rank-contiguous cut of the flat buffer at the hinted boundaries (matrix_fsdp/api.py:153-156)
+            planner = partial(hinted_ordered_group_plan, default_granularity="parameter")
     return matrix_fully_shard(
         module,
         world_size=world_size,

@@ -16,7 +16,7 @@ from math import gcd
 
 import torch
 
-from .layout import ShardPlan
+from .layout import MatrixGroupLayout, ShardPlan
 
 
 @dataclass(frozen=True)
@@ -121,10 +121,12 @@ def shard_sizes_to_matrix_local_units(shard_sizes: tuple[int, ...]) -> tuple[int
     return tuple(size // divisor for size in shard_sizes)
 
 
-def explain_matrix_shard_compatibility(plan: ShardPlan) -> PlacementCompatibility:
-    """A plan is a ``MatrixShard`` when every non-empty rank holds exactly one
-    segment and the segments tile the flat buffer in rank order
-    (placement.py:177-222)."""
+def explain_matrix_shard_compatibility(plan: ShardPlan | MatrixGroupLayout) -> PlacementCompatibility:
+    """A plan (or group layout) is a ``MatrixShard`` when every non-empty rank
+    holds exactly one segment and the segments tile the flat buffer in rank
+    order (placement.py:177-222)."""
+    if isinstance(plan, MatrixGroupLayout):
+        plan = plan.to_shard_plan()
     if plan.total_numel <= 0:
         return PlacementCompatibility(False, "empty shard plans cannot be represented as matrix placements")
     cursor = 0
@@ -157,11 +159,13 @@ def explain_matrix_shard_compatibility(plan: ShardPlan) -> PlacementCompatibilit
     return PlacementCompatibility(True)
 
 
-def is_matrix_shard_compatible_plan(plan: ShardPlan) -> bool:
+def is_matrix_shard_compatible_plan(plan: ShardPlan | MatrixGroupLayout) -> bool:
     return explain_matrix_shard_compatibility(plan).compatible
 
 
-def matrix_shard_from_plan(plan: ShardPlan, *, dims: tuple[int, ...] = (0,)) -> MatrixShard:
+def matrix_shard_from_plan(plan: ShardPlan | MatrixGroupLayout, *, dims: tuple[int, ...] = (0,)) -> MatrixShard:
+    if isinstance(plan, MatrixGroupLayout):
+        plan = plan.to_shard_plan()
     verdict = explain_matrix_shard_compatibility(plan)
     if not verdict.compatible:
         raise ValueError(
@@ -169,3 +173,7 @@ def matrix_shard_from_plan(plan: ShardPlan, *, dims: tuple[int, ...] = (0,)) -> 
             f"Reason: {verdict.reason}."
         )
     return MatrixShard(dims, shard_sizes_to_matrix_local_units(plan.shard_sizes))
+
+
+def matrix_shard_from_layout(layout: MatrixGroupLayout, *, dims: tuple[int, ...] = (0,)) -> MatrixShard:
+    return matrix_shard_from_plan(layout.to_shard_plan(), dims=dims)

@@ -168,6 +168,12 @@ class MixedMuonAdamWOptimizer:
         self.flat_buffers = list(flat_buffers or ())
         self.muon = None
         self.adamw = None
+        with _without_auto_prepare():  # this wrapper drives the units' lifecycle itself
+            self._build(lr, weight_decay, muon_lr, adamw_lr, adamw_betas, adamw_eps, adamw_weight_decay, muon_weight_decay, muon_momentum, muon_ns_steps, muon_adjust_lr_fn)
+        if self.muon is None and self.adamw is None:
+            raise RuntimeError("MixedMuonAdamWOptimizer requires at least one non-empty parameter.")
+
+    def _build(self, lr, weight_decay, muon_lr, adamw_lr, adamw_betas, adamw_eps, adamw_weight_decay, muon_weight_decay, muon_momentum, muon_ns_steps, muon_adjust_lr_fn) -> None:
         if self.muon_params:
             self.muon = Muon(
                 self.muon_params,
@@ -185,8 +191,6 @@ class MixedMuonAdamWOptimizer:
                 eps=adamw_eps,
                 weight_decay=weight_decay if adamw_weight_decay is None else adamw_weight_decay,
             )
-        if self.muon is None and self.adamw is None:
-            raise RuntimeError("MixedMuonAdamWOptimizer requires at least one non-empty parameter.")
 
     @property
     def param_groups(self) -> list[dict[str, Any]]:
@@ -272,12 +276,163 @@ def prepare_units_for_step(units, operation: str = "optimizer.step") -> None:
         unit.prepare_for_optimizer_step(operation)
 
 
-def _manage_lifecycle(optimizer: torch.optim.Optimizer, units: list) -> None:
-    """``optimizer.step()`` first finishes pending backwards and insists on
-    sharded parameters, as the reference's prepared optimizers do
-    (matrix_fsdp/optim/wrapper.py:227-241, 957-977)."""
-    if units:
-        optimizer.register_step_pre_hook(lambda opt, args, kwargs: prepare_units_for_step(units))
+class PreparedMatrixOptimizer:
+    """Lifecycle hooks of the units on a regular ``torch.optim`` optimizer, which
+    stays the object the user holds (matrix_fsdp/optim/wrapper.py:99-247):
+    ``step()`` refuses closures and ``no_sync()``, finishes pending backwards,
+    insists on sharded parameters and (opt-in) lays AdamW state out flat;
+    ``zero_grad()`` refuses ``no_sync()`` and afterwards releases the units'
+    reduced gradient shards.  The optimizer gains ``matrix_fsdp`` (this object),
+    ``state_manager``, ``no_sync``, ``refresh_state_dtensors`` and
+    ``validate_local_state_shapes``; ``remove()`` takes everything off again.
+    The reference's scheduler arguments have no counterpart on one device."""
+
+    _ATTRS = ("matrix_fsdp", "state_manager", "no_sync", "refresh_state_dtensors", "validate_local_state_shapes")
+
+    def __init__(self, optimizer: torch.optim.Optimizer, module_or_units, *, flat_adamw_state: bool = False) -> None:
+        self.optimizer = optimizer
+        self._fsdp_param_groups = units_of(module_or_units)
+        self.flat_adamw_state = flat_adamw_state
+        self.state_manager = MatrixFSDPOptimizerStateManager(optimizer, self._fsdp_param_groups)
+        self._original_zero_grad = optimizer.zero_grad
+        self._removed = False
+        self._handles = [optimizer.register_step_pre_hook(self._step_pre_hook)]
+        optimizer.zero_grad = self._zero_grad  # type: ignore[method-assign]
+        optimizer.matrix_fsdp = self  # type: ignore[attr-defined]
+        optimizer.state_manager = self.state_manager  # type: ignore[attr-defined]
+        optimizer.no_sync = self.no_sync  # type: ignore[attr-defined]
+        optimizer.refresh_state_dtensors = self.refresh_state_dtensors  # type: ignore[attr-defined]
+        optimizer.validate_local_state_shapes = self.validate_local_state_shapes  # type: ignore[attr-defined]
+
+    @property
+    def fsdp_param_groups(self) -> list:
+        return self._fsdp_param_groups
+
+    runtime_param_groups = fsdp_param_groups
+
+    def no_sync(self):
+        from ..runtime.param_group import MatrixFSDPNoSync
+
+        return MatrixFSDPNoSync(self._fsdp_param_groups)
+
+    def _refuse_inside_no_sync(self, operation: str) -> None:
+        if any(unit.is_no_sync_active() for unit in self._fsdp_param_groups):
+            raise RuntimeError(f"{operation} cannot run inside no_sync().")
+
+    def _step_pre_hook(self, optimizer, args, kwargs) -> None:
+        if kwargs.get("closure") is not None or (len(args) > 1 and args[1] is not None):
+            raise NotImplementedError("MatrixFSDP prepared optimizers do not support optimizer closures yet.")
+        self._refuse_inside_no_sync("optimizer.step")
+        prepare_units_for_step(self._fsdp_param_groups)
+        if self.flat_adamw_state:
+            initialize_flat_adamw_state(self.optimizer, collect_flat_buffers(self._fsdp_param_groups))
+
+    def _zero_grad(self, *args: Any, **kwargs: Any) -> None:
+        self._refuse_inside_no_sync("optimizer.zero_grad")
+        for unit in self._fsdp_param_groups:
+            if unit._in_backward:
+                unit.finalize_backward()
+        self._original_zero_grad(*args, **kwargs)
+        for unit in self._fsdp_param_groups:
+            if unit.flat_buffer is not None:
+                unit.flat_buffer.clear_local_grad_shard()
+
+    def remove(self) -> None:
+        if self._removed:
+            return
+        for handle in self._handles:
+            handle.remove()
+        self.optimizer.zero_grad = self._original_zero_grad  # type: ignore[method-assign]
+        for attr in self._ATTRS:
+            if attr in vars(self.optimizer):
+                delattr(self.optimizer, attr)
+        self._removed = True
+
+    # state placement metadata
+    def local_state_summary(self) -> dict[str, Any]:
+        return self.state_manager.local_state_summary()
+
+    def local_state_objects(self):
+        return self.state_manager.local_state_objects()
+
+    def local_state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.local_state_dtensors()
+
+    @property
+    def state_objects(self):
+        if not self.state_manager.state_objects:
+            self.state_manager.refresh_state_dtensors()
+        return self.state_manager.state_objects
+
+    @property
+    def state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.refresh_state_dtensors()
+
+    def refresh_state_dtensors(self) -> dict[str, dict[str, Any]]:
+        return self.state_manager.refresh_state_dtensors()
+
+    def validate_local_state_shapes(self) -> None:
+        self.state_manager.validate_local_state_shapes()
+
+
+def prepare_matrix_optimizer(optimizer: torch.optim.Optimizer, module_or_units, **kwargs: Any) -> PreparedMatrixOptimizer:
+    """Hooks the units' lifecycle onto ``optimizer`` (a second call replaces the
+    first; matrix_fsdp/optim/wrapper.py:250-268)."""
+    existing = getattr(optimizer, "matrix_fsdp", None)
+    if isinstance(existing, PreparedMatrixOptimizer):
+        existing.remove()
+    return PreparedMatrixOptimizer(optimizer, module_or_units, **kwargs)
+
+
+_original_optimizer_init = None
+_auto_prepare_suppressed = 0
+
+
+def install_matrix_optimizer_auto_prepare() -> None:
+    """From now on every ``torch.optim.Optimizer`` built over parameters that a
+    unit manages is prepared as by ``prepare_matrix_optimizer`` (the parameters
+    carry a weak reference to their unit).  Installed once per process, by the
+    first unit (matrix_fsdp/optim/wrapper.py:271-322)."""
+    global _original_optimizer_init
+    if _original_optimizer_init is not None:
+        return
+    _original_optimizer_init = torch.optim.Optimizer.__init__
+
+    def optimizer_init(self, *args: Any, **kwargs: Any) -> None:
+        _original_optimizer_init(self, *args, **kwargs)
+        if _auto_prepare_suppressed or isinstance(getattr(self, "matrix_fsdp", None), PreparedMatrixOptimizer):
+            return
+        units, seen = [], set()
+        for group in self.param_groups:
+            for param in group.get("params", ()):
+                ref = getattr(param, "_matrix_fsdp_param_group_ref", None)
+                unit = ref() if ref is not None else None
+                if unit is not None and id(unit) not in seen:
+                    seen.add(id(unit))
+                    units.append(unit)
+        if units:
+            prepare_matrix_optimizer(self, units)
+
+    torch.optim.Optimizer.__init__ = optimizer_init  # type: ignore[method-assign]
+
+
+def uninstall_matrix_optimizer_auto_prepare() -> None:
+    global _original_optimizer_init
+    if _original_optimizer_init is not None:
+        torch.optim.Optimizer.__init__ = _original_optimizer_init  # type: ignore[method-assign]
+        _original_optimizer_init = None
+
+
+class _without_auto_prepare:
+    """Optimizers built inside belong to a wrapper that manages the lifecycle itself."""
+
+    def __enter__(self) -> None:
+        global _auto_prepare_suppressed
+        _auto_prepare_suppressed += 1
+
+    def __exit__(self, *exc) -> None:
+        global _auto_prepare_suppressed
+        _auto_prepare_suppressed -= 1
 
 
 def make_mixed_muon_adamw_optimizer(module_or_units, *, default_matrix_optimizer: str = "muon", default_other_optimizer: str = "adamw", **optimizer_kwargs: Any) -> MixedMuonAdamWOptimizer:
@@ -324,16 +479,19 @@ def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig 
             module_or_units, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer, **optimizer_kwargs
         )
     params = _local_params(module_or_units)
-    if kind == "adamw":
-        built = FusedAdamW(params, **optimizer_kwargs)
-    elif kind == "sgd":
-        built = torch.optim.SGD(params, **optimizer_kwargs)
-    elif kind == "muon":
-        built = Muon(params, **optimizer_kwargs)
-    else:
-        built = None
+    with _without_auto_prepare():  # prepared below, for the units of module_or_units
+        if kind == "adamw":
+            built = FusedAdamW(params, **optimizer_kwargs)
+        elif kind == "sgd":
+            built = torch.optim.SGD(params, **optimizer_kwargs)
+        elif kind == "muon":
+            built = Muon(params, **optimizer_kwargs)
+        else:
+            built = None
     if built is not None:
-        _manage_lifecycle(built, units_of(module_or_units))
+        units = units_of(module_or_units)
+        if units:
+            prepare_matrix_optimizer(built, units)
         return built
     raise ValueError(f"optimizer must be one of 'adamw', 'sgd', 'muon', or 'mixed_muon_adamw', got {kind!r}.")
 

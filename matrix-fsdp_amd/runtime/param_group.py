@@ -18,6 +18,7 @@ pointing into the reduced local gradient shard.
 """
 from __future__ import annotations
 
+import weakref
 from enum import Enum
 from itertools import count
 from typing import Callable, Iterable, Mapping
@@ -27,7 +28,7 @@ from torch import nn
 from torch.autograd import Variable
 
 from ..core.layout import MatrixGroupLayout, ParamSegment, ShardPlan
-from ..core.managed_param import ManagedParam, ParamShardHint, managed_params_from_module
+from ..core.managed_param import ManagedParam, ManagedParamRegistry, ParamShardHint, managed_params_from_module
 from ..core.plans import contiguous_even_plan, fsdp2_chunk_plan
 from .flat_buffer import MatrixFlatBuffer
 from .grad_bucket import BucketParamGrad, MatrixGradBucket
@@ -177,6 +178,8 @@ class MatrixFSDPParamGroup:
         if not self.managed_params:
             return
         plan = self.planner(self.managed_params, self.world_size)
+        if isinstance(plan, MatrixGroupLayout):  # the group planners hand back the layout form
+            plan = plan.to_shard_plan()
         if len(plan.shard_sizes) != self.world_size:
             raise ValueError(f"planner returned a plan for {len(plan.shard_sizes)} ranks, expected {self.world_size}.")
         self.shard_plan = plan
@@ -186,13 +189,18 @@ class MatrixFSDPParamGroup:
         )
         buffers = list(getattr(self.module, "_matrix_fsdp_flat_buffers", ()))
         self.module._matrix_fsdp_flat_buffers = (*buffers, self.flat_buffer)  # type: ignore[attr-defined]
+        me = weakref.ref(self)
         for mp in self.managed_params:
             setattr(mp.param, _MANAGED_ATTR, True)
+            mp.param._matrix_fsdp_param_group_ref = me  # lets optimizers built over the parameter find their unit
             self._expected_param_ids.add(id(mp.param))
             self._handles.append(mp.param.register_post_accumulate_grad_hook(self._post_accumulate_grad))
         self._handles.append(self.module.register_forward_pre_hook(self._pre_forward, with_kwargs=True))
         self._handles.append(self.module.register_forward_hook(self._post_forward, with_kwargs=True))
         self._record("init")
+        from ..optim.wrapper import install_matrix_optimizer_auto_prepare
+
+        install_matrix_optimizer_auto_prepare()
 
     def _record(self, event: str) -> None:
         self.events.append(event)
@@ -206,6 +214,23 @@ class MatrixFSDPParamGroup:
         segments per rank included), so it equals ``group_layout``: nothing is
         flat-reordered."""
         return self.group_layout
+
+    @property
+    def param_registry(self) -> ManagedParamRegistry:
+        return ManagedParamRegistry(tuple(self.managed_params))
+
+    @property
+    def runtime_layout_compatibility(self):
+        """How the reference's runtime would classify this unit's layout:
+        ``mode`` is ``matrix_shard``, ``segment_runtime``, ``flat_reorder`` or
+        ``unsupported`` (matrix_fsdp/planning/layout_validator.py:33-88).  This
+        runtime executes every valid plan through one segment program, so the
+        verdict is information, not a gate."""
+        from ..planning.layout_validator import explain_runtime_layout_compatibility
+
+        if self.group_layout is None:
+            return None
+        return explain_runtime_layout_compatibility(self.group_layout, self.managed_params, self.world_size)
 
     def owner_ranks(self, fqn: str) -> tuple[int, ...]:
         return self.group_layout.owner_ranks(fqn)

@@ -215,8 +215,9 @@ def test_gradients_accumulate_over_backwards_until_zero_grad(world, rank):
         return torch.cat([full[s.global_start : s.global_end] for s in unit.flat_buffer.local_segments])
 
     prefixed = [(f"blocks.{i}.", u) for i, u in enumerate(units[:-1])] + [("", units[-1])]
-    data = batches(4, seed=9)
-    for round_, zero in enumerate(("none", "zeros")):
+    data = batches(6, seed=9)
+    zeroed_in_place = False
+    for round_, zero in enumerate(("none", "zeros", "none")):
         for micro, (x, y) in enumerate(data[2 * round_ : 2 * round_ + 2]):
             torch.nn.functional.mse_loss(model(x), y).backward()
             torch.nn.functional.mse_loss(twin(x), y).backward()
@@ -224,14 +225,19 @@ def test_gradients_accumulate_over_backwards_until_zero_grad(world, rank):
                 fb = unit.flat_buffer
                 assert torch.equal(fb.local_grad_shard, twin_local_grads(unit)), (round_, micro)
                 assert all(v.managed_param.param.grad.data_ptr() == fb.local_grad_shard.data_ptr() + v.shard_start * 4 for v in fb.local_param_views)
-                assert ("accumulate_local_grad_shard" in unit.events[-3:]) == (micro == 1)
+                # a shard zeroed in place is still live: the next backward adds to the zeros
+                assert ("accumulate_local_grad_shard" in unit.events[-3:]) == (micro == 1 or zeroed_in_place)
+            zeroed_in_place = False
         # no step: the parameters of the two models stay identical, so the gradients can be compared bit for bit
-        opt.zero_grad(set_to_none=(zero == "none"))
         twin.zero_grad(set_to_none=(zero == "none"))
-        if zero == "none":
+        if zero == "none":  # through the optimizer: grads dropped and the reduced shards released
+            opt.zero_grad()
             assert all(p.grad is None for p in model.parameters())
-        else:
+            assert all(u.flat_buffer.local_grad_shard is None for u in units)
+        else:  # through the module: grads zeroed where they are
+            model.zero_grad(set_to_none=False)
             assert all(float(u.flat_buffer.local_grad_shard.abs().sum()) == 0.0 for u in units)
+            zeroed_in_place = True
 
 
 class CheckpointedNet(Net):
@@ -457,3 +463,156 @@ def test_muon_optimizer_policy_in_a_simulated_world_of_two():
             assert rel(p.detach().float().cpu() - start[n], want - start[n]) < tol, n
         else:
             assert p.numel() == 0, n
+
+
+def test_shard0_placement_maps_to_leading_dimension_hints():
+    """The expectations of the reference's test (test/fsdp/test_matrix_fsdp_e2e.py:252-291): a matrix may be cut
+    between rows, a vector between elements, ignored parameters are not asked about, the layout is one stretch per
+    rank."""
+    from torch.distributed.tensor import Shard
+
+    model = nn.Sequential(nn.Linear(4, 2), nn.LayerNorm(2)).to(DEV)
+    assert fully_shard(model, shard_placement_fn=lambda p: Shard(0)) is model
+    unit = model._matrix_fsdp_param_group
+    assert unit.param_registry.param("0.weight").shard_hint == ParamShardHint(split_granularity="row_block", block_shape=(1, 4))
+    assert unit.param_registry.param("0.bias").shard_hint == ParamShardHint(split_granularity="block", block_shape=(1,))
+    assert unit.group_layout is not None and unit.runtime_layout_compatibility.mode == "matrix_shard"
+
+    model = nn.Sequential(nn.Linear(4, 2), nn.LayerNorm(2)).to(DEV)
+    ignored, asked = model[1].weight, []
+
+    def placement(param):
+        asked.append(id(param))
+        return Shard(0)
+
+    fully_shard(model, shard_placement_fn=placement, ignored_params={ignored}, world_size=2, rank=1)
+    unit = model._matrix_fsdp_param_group
+    assert id(ignored) not in asked and "1.weight" not in unit.param_registry.fqns
+    assert unit.param_registry.param("1.bias").shard_hint == ParamShardHint(split_granularity="block", block_shape=(1,))
+    assert unit.shard_plan.shard_sizes == (8, 4)  # 12 elements: the cut nearest to 6 that takes a block on a tie
+
+    seen = []
+    model = nn.Sequential(nn.Linear(4, 2), nn.Linear(2, 1)).to(DEV)
+    fully_shard(model, shard_placement_fn=lambda p: seen.append(id(p)))
+    assert seen == [id(p) for p in model.parameters()]
+
+
+@pytest.mark.parametrize("rank", [0, 1, 2])
+def test_shard0_units_train_like_eager_in_a_simulated_world_of_three(rank):
+    """Every unit is cut at row boundaries into three rank-contiguous stretches (``hinted_ordered_group_plan``);
+    parameters straddling a cut are 1-D slices for the optimizer.  The twin trains whole and then takes back
+    every element outside the rank's stretch."""
+    from torch.distributed.tensor import Shard
+
+    world = 3
+    model, twin = make_pair(seed=11)
+    shard_all(model, world_size=world, rank=rank, shard_placement_fn=lambda p: Shard(0))
+    units = [m._matrix_fsdp_param_group for m in [*model.blocks, model]]
+    twin_params = dict(twin.named_parameters())
+    prefixes = [f"blocks.{i}." for i in range(len(model.blocks))] + [""]
+    for unit in units:
+        assert unit.runtime_layout_compatibility.mode == "matrix_shard"
+        for mp in unit.managed_params:  # cuts fall between rows
+            for piece in unit.group_layout.param(mp.fqn).segments:
+                row = mp.shape[-1] if len(mp.shape) == 2 else 1
+                assert (piece.global_start - mp.offset) % row == 0 and (piece.global_end - mp.offset) % row == 0
+    opt = configure_optimizer(model, "adamw", lr=1e-3, weight_decay=0.1)
+    ref = torch.optim.AdamW(twin.parameters(), lr=1e-3, weight_decay=0.1, foreach=False)
+
+    def stretch(unit, prefix):
+        """(twin parameter, first, last) for the part of each parameter inside the rank's stretch."""
+        lo, hi = unit.shard_plan.local_range(rank)
+        for mp in unit.managed_params:
+            a, b = max(lo, mp.offset), min(hi, mp.end)
+            yield twin_params[prefix + mp.fqn], mp, max(a - mp.offset, 0), max(b - mp.offset, 0)
+
+    for x, y in batches(3, seed=12):
+        torch.nn.functional.mse_loss(model(x), y).backward()
+        opt.step()
+        opt.zero_grad()
+        before = {name: p.detach().clone() for name, p in twin_params.items()}
+        torch.nn.functional.mse_loss(twin(x), y).backward()
+        ref.step()
+        ref.zero_grad()
+        with torch.no_grad():
+            for unit, prefix in zip(units, prefixes):
+                for p, mp, a, b in stretch(unit, prefix):
+                    mine = p.view(-1)[a:b].clone()
+                    p.copy_(before[prefix + mp.fqn])
+                    p.view(-1)[a:b] = mine
+    for unit, prefix in zip(units, prefixes):
+        for p, mp, a, b in stretch(unit, prefix):
+            local = mp.param.detach().view(-1)
+            assert local.numel() == max(b - a, 0), mp.fqn
+            if b > a:
+                assert rel(local.cpu(), p.detach().view(-1)[a:b].cpu()) < 2e-6, mp.fqn
+        unit.unshard()
+        assert unit.flat_buffer.param_data_alias_full_buffer()
+        for mp in unit.managed_params:
+            assert rel(mp.param.detach().cpu(), twin_params[prefix + mp.fqn].detach().cpu()) < 2e-6, mp.fqn
+        unit.reshard()
+
+
+def test_plain_torch_optimizers_are_prepared_automatically():
+    """A ``torch.optim`` optimizer built over a unit's parameters gets the unit's lifecycle hooks by itself
+    (the reference's behaviour, test/fsdp/test_matrix_fsdp_e2e.py:1818-1893, 2006-2022)."""
+    from matrix_fsdp_amd import PreparedMatrixOptimizer, matrix_fully_shard, prepare_matrix_optimizer
+
+    torch.manual_seed(0)
+    model = matrix_fully_shard(nn.Linear(4, 2).to(DEV))
+    unit = model._matrix_fsdp_param_group
+    optimizer = torch.optim.AdamW(model.parameters(), lr=0.01)
+    prepared = optimizer.matrix_fsdp
+    assert isinstance(prepared, PreparedMatrixOptimizer) and optimizer.state_manager is prepared.state_manager
+    model(torch.randn(3, 4, device=DEV)).sum().backward()
+    optimizer.step()
+    assert prepared.state_objects and optimizer.matrix_fsdp.state_objects
+    prepared.validate_local_state_shapes()
+    assert unit.flat_buffer.local_grad_shard is not None
+    optimizer.zero_grad()
+    assert unit.flat_buffer.local_grad_shard is None
+    with pytest.raises(NotImplementedError, match="closures"):
+        optimizer.step(lambda: None)
+    again = prepare_matrix_optimizer(optimizer, model)  # replaces the first preparation
+    assert optimizer.matrix_fsdp is again and prepared._removed
+    again.remove()
+    assert not hasattr(optimizer, "matrix_fsdp") and not hasattr(optimizer, "state_manager")
+    optimizer.zero_grad()  # the class's own method again
+
+    # no_sync on the optimizer: neither step nor zero_grad inside it
+    optimizer = torch.optim.SGD(model.parameters(), lr=0.1)
+    with optimizer.no_sync():
+        with pytest.raises(RuntimeError, match="cannot run inside no_sync"):
+            optimizer.step()
+        with pytest.raises(RuntimeError, match="cannot run inside no_sync"):
+            optimizer.zero_grad()
+    assert not unit.is_no_sync_active()
+
+    # optimizers over foreign parameters are left alone; wrappers keep their inner optimizers unprepared
+    assert not hasattr(torch.optim.SGD(nn.Linear(2, 2).parameters(), lr=0.1), "matrix_fsdp")
+    mixed = configure_optimizer(model, "mixed_muon_adamw", lr=0.01)
+    assert all(not hasattr(opt, "matrix_fsdp") for _, opt in mixed.iter_named_optimizers())
+    assert isinstance(configure_optimizer(model, "adamw", lr=0.01).matrix_fsdp, PreparedMatrixOptimizer)
+
+    muon = torch.optim.Muon(matrix_fully_shard(nn.Linear(4, 2, bias=False).to(DEV)).parameters(), lr=0.01)
+    assert isinstance(muon.matrix_fsdp, PreparedMatrixOptimizer)
+
+
+@pytest.mark.parametrize("set_to_none", [True, False])
+def test_auto_prepared_sgd_matches_eager_over_several_steps(set_to_none):
+    from matrix_fsdp_amd import PreparedMatrixOptimizer
+
+    model, twin = make_pair(seed=21)
+    shard_all(model, world_size=1, rank=0)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9)
+    ref = torch.optim.SGD(twin.parameters(), lr=0.1, momentum=0.9)
+    assert isinstance(opt.matrix_fsdp, PreparedMatrixOptimizer) and len(opt.matrix_fsdp.fsdp_param_groups) == 3
+    for x, y in batches(3, seed=22):
+        for net, optimizer in ((model, opt), (twin, ref)):
+            torch.nn.functional.mse_loss(net(x), y).backward()
+            optimizer.step()
+            optimizer.zero_grad(set_to_none=set_to_none)
+        assert all(unit.flat_buffer.local_grad_shard is None for unit in opt.matrix_fsdp.fsdp_param_groups)
+    ours, theirs = named_full_params(model), named_full_params(twin)
+    for name in theirs:
+        assert rel(ours[name], theirs[name]) < 2e-6, name

@@ -223,8 +223,13 @@ def test_fully_shard_host_rules():
         fully_shard(module)
     with pytest.raises(ValueError, match="floating-point"):
         validate_mixed_precision_policy(MixedPrecisionPolicy(reduce_dtype=torch.int64))
-    with pytest.raises(TypeError, match="ParamShardHint"):
-        fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: "muon")
+    # placements other than Shard(0) are refused as in the reference (matrix_fsdp/api.py:139-149)
+    from torch.distributed.tensor import Replicate, Shard
+
+    with pytest.raises(NotImplementedError, match="only None or torch.distributed.tensor.Shard"):
+        fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: Replicate())
+    with pytest.raises(NotImplementedError, match="supports only Shard\\(0\\)"):
+        fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: Shard(1))
     # wrap policies decide before anything touches the device
     from matrix_fsdp_amd import matrix_fully_shard
     from matrix_fsdp_amd.policy import module_type_policy
