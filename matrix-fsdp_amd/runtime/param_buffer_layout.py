@@ -3,13 +3,18 @@
 One descriptor stands in for the reference's ``StaticParamBufferLayout``
 (matrix_fsdp/runtime/static_param_buffer.py:9-88) and
 ``ElasticParamBufferLayout`` (runtime/elastic_param_buffer.py:111-214), which
-share these properties; only the arithmetic is kept (no caches or pools).
+share these properties (both names are bound to it); only the arithmetic is
+kept (no caches or pools).  ``build_communication_plan`` precomputes what an
+exchange of the layout's shards walks over: the segments, the same with
+neighbours merged, one chunk per segment, and the rank-chunk sizes when every
+rank holds a single stretch (elastic_param_buffer.py:17-81, 197-214).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
 
 from ..core.layout import LayoutSegment, ShardPlan
+from ..kernels.segment_fusion import coalesce_rank_segments
 
 RankSegments = tuple[tuple[LayoutSegment, ...], ...]
 
@@ -57,6 +62,82 @@ def packed_rank_shards_are_full_tensor_order(total_numel: int, shard_sizes, rank
             return False
         base += shard_sizes[rank]
     return True
+
+
+def rank_segments_from_shard_sizes(shard_sizes) -> RankSegments:
+    """One stretch per non-empty rank, in rank order (elastic_param_buffer.py:506-515)."""
+    cursor, out = 0, []
+    for size in shard_sizes:
+        out.append((LayoutSegment(cursor, cursor + size, 0),) if size else ())
+        cursor += size
+    return tuple(out)
+
+
+@dataclass(frozen=True)
+class ElasticRankChunk:
+    rank: int
+    global_start: int
+    global_end: int
+    local_start: int = 0
+
+    @property
+    def numel(self) -> int:
+        return self.global_end - self.global_start
+
+    def as_segment(self) -> LayoutSegment:
+        return LayoutSegment(self.global_start, self.global_end, self.local_start)
+
+
+@dataclass(frozen=True)
+class ElasticCommunicationPlan:
+    rank_segments: RankSegments
+    coalesced_rank_segments: RankSegments
+    rank_chunks: tuple[ElasticRankChunk, ...]
+    rank_chunk_shard_sizes: tuple[int, ...] | None
+    rank_chunk_segments: RankSegments | None
+    rank_chunk_fast_path: bool
+    packed_full_order: bool
+
+    @property
+    def world_size(self) -> int:
+        return len(self.rank_segments)
+
+    @property
+    def segment_count(self) -> int:
+        return sum(len(s) for s in self.rank_segments)
+
+    @property
+    def coalesced_segment_count(self) -> int:
+        return sum(len(s) for s in self.coalesced_rank_segments)
+
+    @property
+    def max_segments_per_rank(self) -> int:
+        return max((len(s) for s in self.rank_segments), default=0)
+
+    @property
+    def max_coalesced_segments_per_rank(self) -> int:
+        return max((len(s) for s in self.coalesced_rank_segments), default=0)
+
+    @property
+    def rank_chunk_count(self) -> int:
+        return len(self.rank_chunks)
+
+    @property
+    def nonempty_rank_chunk_count(self) -> int:
+        return sum(1 for chunk in self.rank_chunks if chunk.numel > 0)
+
+    def as_summary(self) -> dict[str, object]:
+        return {
+            "communication_plan_segment_count": self.segment_count,
+            "communication_plan_coalesced_segment_count": self.coalesced_segment_count,
+            "communication_plan_max_segments_per_rank": self.max_segments_per_rank,
+            "communication_plan_max_coalesced_segments_per_rank": self.max_coalesced_segments_per_rank,
+            "communication_plan_rank_chunk_count": self.rank_chunk_count,
+            "communication_plan_nonempty_rank_chunk_count": self.nonempty_rank_chunk_count,
+            "communication_plan_rank_chunk_fast_path": self.rank_chunk_fast_path,
+            "communication_plan_packed_full_order": self.packed_full_order,
+            "communication_plan_has_rank_chunk_shard_sizes": self.rank_chunk_shard_sizes is not None,
+        }
 
 
 @dataclass(frozen=True)
@@ -125,6 +206,19 @@ class ParamBufferLayout:
         or padded ``W * max_shard``."""
         return self.total_shard_numel if compact else self.padded_numel
 
+    def build_communication_plan(self) -> ElasticCommunicationPlan:
+        segments = self.rank_segments or rank_segments_from_shard_sizes(self.shard_sizes)
+        chunk_sizes = rank_chunk_shard_sizes(segments)
+        return ElasticCommunicationPlan(
+            rank_segments=segments,
+            coalesced_rank_segments=coalesce_rank_segments(segments),
+            rank_chunks=tuple(ElasticRankChunk(rank, s.global_start, s.global_end, s.local_start) for rank, segs in enumerate(segments) for s in segs),
+            rank_chunk_shard_sizes=chunk_sizes,
+            rank_chunk_segments=None if chunk_sizes is None else rank_segments_from_shard_sizes(chunk_sizes),
+            rank_chunk_fast_path=chunk_sizes is not None,
+            packed_full_order=self.packed_rank_shards_are_full_tensor_order,
+        )
+
     def as_summary(self) -> dict[str, object]:
         return {
             "rank_chunk_fast_path": self.rank_chunk_fast_path,
@@ -138,3 +232,7 @@ class ParamBufferLayout:
             "padding_waste_ratio": self.padding_waste_ratio,
             "owner_imbalance_ratio": self.owner_imbalance_ratio,
         }
+
+
+StaticParamBufferLayout = ParamBufferLayout
+ElasticParamBufferLayout = ParamBufferLayout

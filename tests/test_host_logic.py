@@ -101,6 +101,33 @@ def test_param_buffer_layout_reference_vectors(golden):
     assert not layout.rank_chunk_fast_path and not layout.packed_rank_shards_are_full_tensor_order
 
 
+def test_communication_plan_reference_expectations():
+    """test/fsdp/test_elastic_param_buffer.py:32-82: the plan keeps the layout's segments, merges neighbours, lists
+    one chunk per segment and knows the rank-chunk sizes exactly when every rank holds one stretch in rank order."""
+    from matrix_fsdp_amd.core.layout import LayoutSegment as S
+    from matrix_fsdp_amd.runtime.param_buffer_layout import ElasticCommunicationPlan, ElasticParamBufferLayout, StaticParamBufferLayout
+
+    assert StaticParamBufferLayout is ParamBufferLayout and ElasticParamBufferLayout is ParamBufferLayout
+    rank_segments = ((S(0, 4, 0),), (S(4, 10, 0),), ())
+    plan = ElasticParamBufferLayout(10, (4, 6, 0), rank_segments).build_communication_plan()
+    assert isinstance(plan, ElasticCommunicationPlan) and plan.rank_segments is rank_segments
+    assert plan.rank_chunk_shard_sizes == (4, 6, 0) and plan.rank_chunk_segments == rank_segments
+    assert plan.rank_chunk_fast_path and plan.packed_full_order
+    assert plan.rank_chunk_count == 2 and plan.nonempty_rank_chunk_count == 2 and plan.world_size == 3
+    assert plan.as_summary()["communication_plan_rank_chunk_fast_path"] is True
+    assert [c.as_segment() for c in plan.rank_chunks] == [S(0, 4, 0), S(4, 10, 0)] and [c.rank for c in plan.rank_chunks] == [0, 1]
+
+    plan = ElasticParamBufferLayout(6, (4, 2), ((S(0, 2, 0), S(2, 4, 2)), (S(4, 6, 0),))).build_communication_plan()
+    assert plan.coalesced_rank_segments == ((S(0, 4, 0),), (S(4, 6, 0),))
+    assert plan.rank_chunk_shard_sizes is None and not plan.rank_chunk_fast_path
+    assert plan.segment_count == 3 and plan.coalesced_segment_count == 2
+    assert plan.max_segments_per_rank == 2 and plan.max_coalesced_segments_per_rank == 1
+
+    # no segment table: the shard sizes alone describe rank-ordered stretches
+    plan = ParamBufferLayout(10, (6, 0, 4), None).build_communication_plan()
+    assert plan.rank_segments == ((S(0, 6, 0),), (), (S(6, 10, 0),)) and plan.rank_chunk_shard_sizes == (6, 0, 4)
+
+
 @pytest.mark.parametrize("case", ["grad_bucket_padded_rank_major", "grad_bucket_flat_cat", "grad_bucket_chunk_cat"])
 def test_classify_copy_in_layout_reference_vectors(golden, case):
     g = golden[case]
