@@ -130,3 +130,55 @@ def test_default_shard_hint_rules():
     assert custom["block.q.weight"] == adamw and custom["table"] == muon
     with pytest.raises(ValueError, match="unknown parameters: nope"):
         build_shard_hints(Model(), overrides={"nope": muon})
+
+
+def test_moe_hint_rules_and_expert_planner():
+    """test/fsdp/test_shard_hint.py:68-110: rule names in order, experts and router recognised by module path; the
+    hinted experts then stay together under ``expert_owner_tail_plan`` and pass the layout validator."""
+    from matrix_fsdp_amd.core.managed_param import ManagedParamRegistry, ParamRuntimeKind
+    from matrix_fsdp_amd.planning import default_shard_hint_rules, expert_owner_tail_plan, validate_group_layout
+
+    assert tuple(rule.name for rule in default_shard_hint_rules()) == (
+        "moe_expert_owner", "router", "muon_linear_weight", "no_split_embedding", "no_split_norm", "no_split_bias", "no_split_1d",
+    )
+
+    class Expert(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.w1 = nn.Linear(4, 8, bias=True)
+            self.w2 = nn.Linear(8, 4, bias=False)
+
+    class MoEBlock(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.router = nn.Linear(4, 2, bias=False)
+            self.experts = nn.ModuleList([Expert(), Expert(), Expert()])
+            self.norm = nn.LayerNorm(4)
+
+    class Model(nn.Module):
+        def __init__(self) -> None:
+            super().__init__()
+            self.moe = MoEBlock()
+            self.experts = nn.Linear(4, 4)  # no expert index below it: an ordinary linear layer
+
+    model = Model()
+    hints = build_shard_hints(model)
+    assert hints["moe.experts.0.w1.weight"] == ParamShardHint(
+        optimizer_type="muon", split_granularity="matrix_owner", runtime_kind=ParamRuntimeKind.EXPERT_OWNER, parallel_role="routed_expert", expert_id=0, expert_group_id="moe.experts.0"
+    )
+    assert hints["moe.experts.0.w1.bias"] == ParamShardHint(
+        optimizer_type="adamw", split_granularity="parameter", runtime_kind=ParamRuntimeKind.EXPERT_OWNER, parallel_role="routed_expert", expert_id=0, expert_group_id="moe.experts.0"
+    )
+    assert hints["moe.experts.1.w2.weight"].expert_group_id == "moe.experts.1" and hints["moe.experts.2.w2.weight"].expert_id == 2
+    assert hints["moe.router.weight"] == ParamShardHint(optimizer_type="adamw", split_granularity="parameter", runtime_kind=ParamRuntimeKind.FSDP_GATHER, parallel_role="router")
+    assert hints["experts.weight"] == ParamShardHint(optimizer_type="muon", split_granularity="matrix_owner")
+    assert hints["moe.norm.weight"] == ParamShardHint(optimizer_type="adamw", split_granularity="parameter")
+
+    params = ManagedParamRegistry.from_module(model, shard_hints=hints).as_list()
+    layout = expert_owner_tail_plan(params, 2)
+    validate_group_layout(layout, params, 2)  # includes: one owner rank per expert group
+    owners = {group: {layout.owner_ranks(p.fqn) for p in params if p.shard_hint.expert_group_id == group} for group in ("moe.experts.0", "moe.experts.1", "moe.experts.2")}
+    assert all(len(ranks) == 1 for ranks in owners.values())
+    # three experts of 72 elements: ranks 0, 1, 0; the dense tail (16 + 8 + 4 + 4 + 4), largest first, all fits on rank 1
+    assert layout.shard_sizes == (144, 108)
+    assert layout.owner_ranks("moe.experts.2.w1.bias") == (0,) and layout.owner_ranks("moe.router.weight") == (1,)
