@@ -63,6 +63,8 @@ def matrix_fully_shard(
     wrap_policy: WrapPolicy | None = None,
     auto_shard_hints: bool = False,
     auto_planner_policy: str | None = None,
+    use_saved_tensor_hooks: bool = True,
+    full_param_buffer_pool=None,
 ) -> nn.Module:
     """Turns ``module`` into one unit: its parameters (those no nested unit
     manages yet) move into a flat buffer sharded by ``planner`` for the
@@ -75,7 +77,10 @@ def matrix_fully_shard(
     ``auto_shard_hints`` derives the hints from the module structure;
     ``auto_planner_policy="muon_shard_aware"`` keeps every parameter whole on
     an owner rank (the other planner families of the reference do not exist
-    here)."""
+    here).  ``use_saved_tensor_hooks`` (default on, as in the reference) keeps
+    autograd from pinning a unit's full buffer between forward and backward;
+    ``full_param_buffer_pool`` (a ``FullParamBufferPool``) lets units of equal
+    size unshard into the same storage."""
     validate_mixed_precision_policy(mp_policy)
     if not isinstance(reshard_after_forward, bool):
         # an int asks for resharding to a smaller world after forward (matrix_fsdp/runtime/fsdp_unit.py:1705-1720)
@@ -96,6 +101,8 @@ def matrix_fully_shard(
         reduce_dtype=getattr(mp_policy, "reduce_dtype", None),
         output_dtype=getattr(mp_policy, "output_dtype", None),
         cast_forward_inputs=getattr(mp_policy, "cast_forward_inputs", True),
+        use_saved_tensor_hooks=use_saved_tensor_hooks,
+        full_param_buffer_pool=full_param_buffer_pool,
     )
     if wrap_policy is not None:
         if shard_hints is not None:

@@ -72,6 +72,7 @@ class MatrixFlatBuffer:
         param_dtype: torch.dtype | None = None,
         reduce_dtype: torch.dtype | None = None,
         keep_world_shards: bool = True,
+        full_param_buffer_pool=None,
     ) -> None:
         if not managed_params:
             raise ValueError("MatrixFlatBuffer needs at least one parameter.")
@@ -111,6 +112,8 @@ class MatrixFlatBuffer:
         self.world_shards: torch.Tensor | None = world if keep_world_shards else None
         self.local_shard = world[self.local_start : self.local_end] if keep_world_shards else world[self.local_start : self.local_end].clone()
         self.full_buffer: torch.Tensor | None = None
+        self.full_param_buffer_pool = full_param_buffer_pool
+        self._full_buffer_pooled = False
         self.local_grad_shard: torch.Tensor | None = None
         self.grad_bucket_input: torch.Tensor | None = None
         self.grad_bucket_input_is_compact = False
@@ -239,7 +242,7 @@ class MatrixFlatBuffer:
                 view = views[0]
                 data = self.local_shard[view.shard_start : view.shard_end]
                 mp.param.data = data.view(mp.shape) if view.numel == mp.numel else data
-        self.full_buffer = None
+        self.clear_full_params()
 
     def use_full_param_buffer(self) -> None:
         """``param.data`` -> zero-copy view of the full buffer (flat_buffer.py:413-425)."""
@@ -282,13 +285,20 @@ class MatrixFlatBuffer:
         """Materialises the full buffer from the gathered padded shards
         (un-pad + unpack fused, one launch) and points every parameter at
         it."""
+        pool = self.full_param_buffer_pool
         if gathered_padded is None:
             gathered_padded = self.gathered_padded_shards()
         dtype = gathered_padded.dtype
+        self.clear_full_params()
+        pooled = False
         if out is None:
-            out = torch.empty(self.plan.total_numel, dtype=dtype, device=self.device)
+            if pool is not None:
+                out, pooled = pool.acquire(gathered_padded, self.plan.total_numel), True
+            else:
+                out = torch.empty(self.plan.total_numel, dtype=dtype, device=self.device)
         self._program("unpack_padded", dtype).run((gathered_padded,), out)
         self.full_buffer = out
+        self._full_buffer_pooled = pooled
         self.use_full_param_buffer()
         return out
 
@@ -337,7 +347,12 @@ class MatrixFlatBuffer:
         self._program("pack_compact", full_tensor.dtype, out_dtype).run((full_tensor,), self.world_shards)
 
     def clear_full_params(self) -> None:
+        """Drops the full buffer; one that came from the pool goes back to it.
+        The parameters must not point into it any more."""
+        if self.full_buffer is not None and self._full_buffer_pooled and self.full_param_buffer_pool is not None:
+            self.full_param_buffer_pool.release(self.full_buffer)
         self.full_buffer = None
+        self._full_buffer_pooled = False
 
     def clear_local_grad_shard(self) -> None:
         self.local_grad_shard = None

@@ -78,6 +78,16 @@ def _tensors_requiring_grad(obj) -> Iterable[torch.Tensor]:
             yield from _tensors_requiring_grad(o)
 
 
+class _FullBufferView:
+    """What autograd keeps in place of a tensor that lives in a unit's full
+    buffer: the view's geometry relative to the buffer's first element."""
+
+    __slots__ = ("shape", "stride", "offset")
+
+    def __init__(self, shape: tuple[int, ...], stride: tuple[int, ...], offset: int) -> None:
+        self.shape, self.stride, self.offset = shape, stride, offset
+
+
 class MatrixFSDPNoSync:
     """``with model.no_sync():`` -- micro-batches whose gradients are to be
     accumulated before the next optimizer step (matrix_fsdp/runtime/fsdp_unit.py:70-97).
@@ -125,9 +135,14 @@ class MatrixFSDPParamGroup:
         reduce_dtype: torch.dtype | None = None,
         output_dtype: torch.dtype | None = None,
         cast_forward_inputs: bool = True,
+        use_saved_tensor_hooks: bool = True,
+        full_param_buffer_pool=None,
     ) -> None:
         if world_size < 1 or not 0 <= rank < world_size:
             raise ValueError(f"rank {rank} is outside a world of {world_size}.")
+        if full_param_buffer_pool is not None and full_param_buffer_pool.max_cached_per_key > 0 and not use_saved_tensor_hooks:
+            # a view autograd saved in the forward would read another unit's values from the shared storage
+            raise ValueError("a full_param_buffer_pool that keeps buffers needs use_saved_tensor_hooks=True.")
         self.module = module
         self.world_size = world_size
         self.rank = rank
@@ -139,6 +154,10 @@ class MatrixFSDPParamGroup:
         self.reduce_dtype = reduce_dtype
         self.output_dtype = output_dtype
         self.cast_forward_inputs = cast_forward_inputs
+        self.use_saved_tensor_hooks = use_saved_tensor_hooks
+        self.full_param_buffer_pool = full_param_buffer_pool
+        self._saved_tensor_contexts: list = []
+        self.saved_full_param_views = 0
         self.managed_params: list[ManagedParam] = []
         self.flat_buffer: MatrixFlatBuffer | None = None
         self.shard_plan: ShardPlan | None = None
@@ -185,7 +204,8 @@ class MatrixFSDPParamGroup:
         self.shard_plan = plan
         self.group_layout = MatrixGroupLayout.from_shard_plan(plan, self.managed_params)
         self.flat_buffer = MatrixFlatBuffer(
-            self.managed_params, plan, self.rank, param_dtype=self.param_dtype, reduce_dtype=self.reduce_dtype
+            self.managed_params, plan, self.rank, param_dtype=self.param_dtype, reduce_dtype=self.reduce_dtype,
+            full_param_buffer_pool=self.full_param_buffer_pool,
         )
         buffers = list(getattr(self.module, "_matrix_fsdp_flat_buffers", ()))
         self.module._matrix_fsdp_flat_buffers = (*buffers, self.flat_buffer)  # type: ignore[attr-defined]
@@ -196,6 +216,8 @@ class MatrixFSDPParamGroup:
             self._expected_param_ids.add(id(mp.param))
             self._handles.append(mp.param.register_post_accumulate_grad_hook(self._post_accumulate_grad))
         self._handles.append(self.module.register_forward_pre_hook(self._pre_forward, with_kwargs=True))
+        # leaves the saved-tensor hooks first, and also when the forward raises
+        self._handles.append(self.module.register_forward_hook(self._leave_saved_tensor_hooks, always_call=True))
         self._handles.append(self.module.register_forward_hook(self._post_forward, with_kwargs=True))
         self._record("init")
         from ..optim.wrapper import install_matrix_optimizer_auto_prepare
@@ -316,10 +338,50 @@ class MatrixFSDPParamGroup:
         self.lifecycle_state = FSDPLifecycleState.SHARDED
         self._record(f"reshard:{reason}")
 
+    # ------------------------------------------------------------------ saved tensors (fsdp_unit.py:1325-1382)
+    # Autograd saves views of the parameters for the backward (``linear`` keeps ``weight.t()``), and such a view
+    # pins the storage it was cut from: a full buffer "freed" after the forward would stay allocated until the
+    # backward, and one handed to another unit through a buffer pool would be read back with that unit's values.
+    # While the unit's forward runs, tensors that live in its full buffer are therefore saved as their geometry
+    # only and rebuilt on the buffer the backward has gathered.  (torch applies only the innermost pair of
+    # saved-tensor hooks, so activation checkpointing around the *inside* of a unit's forward is shadowed there.)
+    def _enter_saved_tensor_hooks(self) -> None:
+        context = None
+        if self.use_saved_tensor_hooks and torch.is_grad_enabled() and not self._single_rank_alias():
+            context = torch.autograd.graph.saved_tensors_hooks(self._pack_saved_tensor, self._unpack_saved_tensor)
+            context.__enter__()
+        self._saved_tensor_contexts.append(context)  # one entry per forward call, so that leaving pairs up
+
+    def _leave_saved_tensor_hooks(self, *unused) -> None:
+        if self.flat_buffer is not None and self._saved_tensor_contexts:
+            context = self._saved_tensor_contexts.pop()
+            if context is not None:
+                context.__exit__(None, None, None)
+
+    def _pack_saved_tensor(self, tensor: torch.Tensor):
+        full = self.flat_buffer.full_buffer
+        if full is None or tensor.dtype != full.dtype or tensor.device != full.device:
+            return tensor
+        if tensor.untyped_storage().data_ptr() != full.untyped_storage().data_ptr():
+            return tensor
+        self.saved_full_param_views += 1
+        return _FullBufferView(tuple(tensor.shape), tuple(tensor.stride()), tensor.storage_offset() - full.storage_offset())
+
+    def _unpack_saved_tensor(self, saved):
+        if not isinstance(saved, _FullBufferView):
+            return saved
+        if self.lifecycle_state != FSDPLifecycleState.UNSHARDED:
+            self.unshard("saved_tensor")
+        full = self.flat_buffer.full_buffer
+        if full is None:
+            raise RuntimeError("Saved full parameter view was unpacked before full parameters were available.")
+        return full.as_strided(saved.shape, saved.stride, full.storage_offset() + saved.offset)
+
     # ------------------------------------------------------------------ forward hooks
     def _pre_forward(self, module, args, kwargs):
         if self.flat_buffer is None:
             return args, kwargs
+        self._enter_saved_tensor_hooks()  # first, so that the always-called leave hook pairs up even if this hook raises
         if self._in_backward:
             # activation checkpointing re-runs the forward in the middle of this unit's backward: the parameters
             # are (or become) full again and the bookkeeping of the backward in flight is left alone

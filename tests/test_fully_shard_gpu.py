@@ -616,3 +616,94 @@ def test_auto_prepared_sgd_matches_eager_over_several_steps(set_to_none):
     ours, theirs = named_full_params(model), named_full_params(twin)
     for name in theirs:
         assert rel(ours[name], theirs[name]) < 2e-6, name
+
+
+class TransposedLinear(nn.Module):
+    """``x @ w.t()`` spelled out: autograd saves the view ``w.t()``, not the parameter."""
+
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.w = nn.Parameter(torch.randn(dim, dim) / dim**0.5)
+
+    def forward(self, x):
+        return torch.tanh(x @ self.w.t())
+
+
+def _stack(dim: int, depth: int, seed: int):
+    torch.manual_seed(seed)
+    model = nn.Sequential(*[TransposedLinear(dim) for _ in range(depth)]).to(DEV)
+    return model, copy.deepcopy(model)
+
+
+def test_saved_tensor_hooks_free_full_buffers_between_forward_and_backward():
+    """Without the hooks the views autograd saved keep every layer's full buffer alive until the backward; with them
+    a resharded layer's buffer is really gone (matrix_fsdp/runtime/fsdp_unit.py:1355-1382).  Gradients are the same
+    either way, and the same as the eager twin's."""
+    from matrix_fsdp_amd import matrix_fully_shard
+
+    dim, depth, world = 512, 6, 4
+    full_bytes = dim * dim * 4
+    held, grads = {}, {}
+    x = torch.randn(8, dim, device=DEV)
+    for hooks in (False, True, False):  # the first pass also pays for the libraries' one-time workspaces
+        model, twin = _stack(dim, depth, seed=3)
+        for layer in model:
+            matrix_fully_shard(layer, world_size=world, rank=1, use_saved_tensor_hooks=hooks)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = model(x)
+        held[hooks] = torch.cuda.memory_allocated() - before
+        out.square().mean().backward()
+        units = [layer._matrix_fsdp_param_group for layer in model]
+        assert all(u.lifecycle_state == FSDPLifecycleState.SHARDED for u in units)
+        # the first layer's input needs no gradient, so its product keeps no view of the weight
+        assert sum(u.saved_full_param_views for u in units) == (depth - 1 if hooks else 0)
+        twin(x).square().mean().backward()
+        for unit, ref_layer in zip(units, twin):
+            want = ref_layer.w.grad.view(-1).chunk(world)[1]  # the other ranks of the simulated world contribute nothing
+            assert rel(unit.flat_buffer.local_grad_shard, want) < 1e-6
+        grads[hooks] = torch.cat([u.flat_buffer.local_grad_shard for u in units])
+    assert torch.equal(grads[True], grads[False])
+    assert held[False] - held[True] >= (depth - 2) * full_bytes, held  # every pinned buffer but (at most) the last layer's
+    assert held[True] < 2 * full_bytes + depth * 8 * dim * 4 * 4, held
+
+
+def test_full_param_buffer_pool_shares_one_buffer_between_equal_units():
+    """Equal layers unshard into the same storage, forward and backward, and still train like the eager twin: what
+    autograd saved of a layer's parameters is rebuilt on the buffer gathered for that layer's backward."""
+    from matrix_fsdp_amd import FullParamBufferPool, matrix_fully_shard
+
+    dim, depth, world = 256, 4, 2
+    pool = FullParamBufferPool(max_cached_per_key=1)
+    model, twin = _stack(dim, depth, seed=4)
+    for layer in model:
+        matrix_fully_shard(layer, world_size=world, rank=0, full_param_buffer_pool=pool)
+    units = [layer._matrix_fsdp_param_group for layer in model]
+    seen = set()
+    for unit in units:
+        unit.unshard()
+        seen.add(unit.flat_buffer.full_buffer.data_ptr())
+        assert unit.flat_buffer.param_data_alias_full_buffer()
+        unit.reshard()
+        assert unit.flat_buffer.full_buffer is None
+    assert len(seen) == 1 and pool.stats()["allocations"] == 1 and pool.stats()["reuses"] == depth - 1
+    opt = configure_optimizer(model, "adamw", lr=1e-2, weight_decay=0.0)
+    ref = torch.optim.AdamW(twin.parameters(), lr=1e-2, weight_decay=0.0, foreach=False)
+    gen = torch.Generator().manual_seed(5)
+    for _ in range(3):
+        x = torch.randn(16, dim, generator=gen).to(DEV)
+        model(x).square().mean().backward()
+        opt.step()
+        opt.zero_grad()
+        before = [p.detach().clone() for p in twin.parameters()]
+        twin(x).square().mean().backward()
+        ref.step()
+        ref.zero_grad()
+        with torch.no_grad():  # the other rank of the simulated world never steps
+            for p, old in zip(twin.parameters(), before):
+                half = p.numel() // world
+                p.view(-1)[half:] = old.view(-1)[half:]
+    for unit, ref_layer in zip(units, twin):
+        assert rel(unit.flat_buffer.local_shard, ref_layer.w.detach().view(-1)[: dim * dim // world]) < 2e-6
+    stats = pool.stats()
+    assert stats["allocations"] <= 2 and stats["reuses"] >= 3 * 2 * depth - 1, stats

@@ -313,3 +313,47 @@ def test_wrap_policies():
             make(linear, object())
     with pytest.raises(TypeError, match="callable"):
         not_policy(object())
+
+
+def test_full_param_buffer_pool_bookkeeping():
+    """test/fsdp/test_flat_buffer.py:277-301 on CPU tensors with a hand-made event: a released buffer is handed
+    out again only once its release event has completed; at most ``max_cached_per_key`` are held per key."""
+    from matrix_fsdp_amd import FullParamBufferPool
+
+    class Event:
+        def __init__(self, complete):
+            self.complete = complete
+
+        def query(self):
+            return self.complete
+
+    pool = FullParamBufferPool(max_cached_per_key=1)
+    buffer = torch.arange(6, dtype=torch.float32)
+    event = Event(False)
+    release = pool.release(buffer, cuda_event=event)
+    assert (release.kind, release.numel, release.bytes) == ("pending_event", 6, 24)
+    stats = pool.stats()
+    assert (stats["cached_buffers"], stats["pending_buffers"], stats["pending_releases"], stats["pending_bytes"]) == (0, 1, 1, 24)
+    assert not pool.can_cache(buffer)  # the waiting one counts
+    assert pool.release(torch.zeros(6), cuda_event=Event(True)).kind == "dropped"
+    fresh = pool.acquire(buffer, 6)
+    assert fresh.data_ptr() != buffer.data_ptr()
+    event.complete = True
+    got = pool.acquire_with_stats(buffer, 6)
+    assert got.reused and got.tensor.data_ptr() == buffer.data_ptr()
+    stats = pool.stats()
+    assert (stats["pending_buffers"], stats["reuses"], stats["allocations"], stats["drops"]) == (0, 1, 1, 1)
+    # keys: device, dtype and element count
+    assert pool.release(buffer).kind == "cached" and pool.release(None).kind == "none"
+    assert not pool.acquire_with_stats(buffer.double(), 6).reused and not pool.acquire_with_stats(buffer, 5).reused
+    assert pool.acquire_with_stats(buffer.view(2, 3), 6).reused
+    pool.release(buffer)
+    pool.clear()
+    assert pool.stats()["cached_buffers"] == 0
+    assert FullParamBufferPool().release(buffer).kind == "dropped"  # a pool of capacity 0 keeps nothing
+    with pytest.raises(ValueError, match="non-negative"):
+        FullParamBufferPool(max_cached_per_key=-1)
+    from matrix_fsdp_amd.runtime.param_group import MatrixFSDPParamGroup
+
+    with pytest.raises(ValueError, match="needs use_saved_tensor_hooks"):
+        MatrixFSDPParamGroup(torch.nn.Linear(2, 2), full_param_buffer_pool=FullParamBufferPool(max_cached_per_key=1), use_saved_tensor_hooks=False)
