@@ -15,6 +15,7 @@ from typing import Callable, Mapping
 
 import torch
 from torch import nn
+from torch.distributed.fsdp import OffloadPolicy
 from torch.distributed.tensor import Shard
 
 from .core.layout import ShardPlan
@@ -149,17 +150,39 @@ def _leading_dim_shard_hint(fqn: str, param: nn.Parameter) -> ParamShardHint:
     return ParamShardHint(split_granularity="block", block_shape=(int(param.numel() // param.shape[0]),))
 
 
+def _refuse_multi_device_arguments(mesh, offload_policy, dp_mesh_dims) -> None:
+    """The reference's arguments for process meshes and host offload are taken
+    in their neutral values only: there is one device and no process group."""
+    if mesh is not None and int(mesh.size()) != 1:
+        raise NotImplementedError(
+            "fully_shard(mesh=...) over several ranks needs a process group, which does not exist here; "
+            "world_size= / rank= shard a unit for a simulated world on the one device."
+        )
+    if dp_mesh_dims is not None:
+        raise NotImplementedError("fully_shard(dp_mesh_dims=...) selects dimensions of a multi-rank mesh, which does not exist here.")
+    if offload_policy is not None:
+        # torch.distributed.fsdp.OffloadPolicy() means "no offload"; CPUOffloadPolicy on a device-resident model is
+        # refused by the reference as well (matrix_fsdp/core/mixed_precision.py:39-56)
+        if not isinstance(offload_policy, OffloadPolicy):
+            raise TypeError(f"offload_policy must be an OffloadPolicy, got {type(offload_policy).__name__}.")
+        if type(offload_policy) is not OffloadPolicy:
+            raise NotImplementedError(f"fully_shard(offload_policy={type(offload_policy).__name__}) is not available: shards stay in device memory.")
+
+
 def fully_shard(
     module: nn.Module,
     *,
-    world_size: int = 1,
-    rank: int = 0,
+    mesh=None,
     reshard_after_forward: bool | None = None,
     shard_placement_fn: Callable[[nn.Parameter], object | None] | None = None,
     mp_policy=_DEFAULT_MP_POLICY,
+    offload_policy=None,
     ignored_params: set[nn.Parameter] | None = None,
-    planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
+    dp_mesh_dims=None,
     optimizer_policy: str | None = None,
+    world_size: int = 1,
+    rank: int = 0,
+    planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
 ) -> nn.Module:
     """FSDP2-style spelling (matrix_fsdp/api.py:213-263): ``shard_placement_fn``
     maps a parameter to ``torch.distributed.tensor.Shard(0)`` or ``None`` (a
@@ -170,7 +193,11 @@ def fully_shard(
     ``"mixed_muon_adamw"``, ...) derives the hints from the module structure
     (``build_shard_hints``) and keeps every parameter whole on an owner rank
     (``MuonOwnerPlanner``; pass one planner object to all units to balance the
-    ranks across units)."""
+    ranks across units).  The first nine parameters are the reference's, in its
+    order; ``mesh`` (a one-rank mesh at most), ``offload_policy`` (no offload)
+    and ``dp_mesh_dims`` (``None``) are accepted in their neutral values, and
+    ``world_size`` / ``rank`` / ``planner`` are this build's additions."""
+    _refuse_multi_device_arguments(mesh, offload_policy, dp_mesh_dims)
     hints: dict[str, ParamShardHint] = {}
     if optimizer_policy is not None:
         policy = optimizer_policy.lower()

@@ -250,6 +250,21 @@ def test_fully_shard_host_rules():
         fully_shard(module)
     with pytest.raises(ValueError, match="floating-point"):
         validate_mixed_precision_policy(MixedPrecisionPolicy(reduce_dtype=torch.int64))
+    # the reference's parameters come first and in its order (test/fsdp/test_matrix_fsdp_e2e.py:206-226)
+    import inspect
+
+    parameters = inspect.signature(fully_shard).parameters
+    assert tuple(parameters)[:9] == ("module", "mesh", "reshard_after_forward", "shard_placement_fn", "mp_policy", "offload_policy", "ignored_params", "dp_mesh_dims", "optimizer_policy")
+    assert all(parameters[name].kind == inspect.Parameter.KEYWORD_ONLY for name in tuple(parameters)[1:])
+    assert parameters["reshard_after_forward"].default is None and parameters["optimizer_policy"].default is None
+    from torch.distributed.fsdp import CPUOffloadPolicy
+
+    with pytest.raises(NotImplementedError, match="CPUOffloadPolicy"):
+        fully_shard(torch.nn.Linear(2, 2), offload_policy=CPUOffloadPolicy())
+    with pytest.raises(TypeError, match="must be an OffloadPolicy"):
+        fully_shard(torch.nn.Linear(2, 2), offload_policy="cpu")
+    with pytest.raises(NotImplementedError, match="dp_mesh_dims"):
+        fully_shard(torch.nn.Linear(2, 2), dp_mesh_dims=(0, 1))
     # placements other than Shard(0) are refused as in the reference (matrix_fsdp/api.py:139-149)
     from torch.distributed.tensor import Replicate, Shard
 
