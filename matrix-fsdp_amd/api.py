@@ -66,6 +66,7 @@ def matrix_fully_shard(
     auto_planner_policy: str | None = None,
     use_saved_tensor_hooks: bool = True,
     full_param_buffer_pool=None,
+    use_zero_copy_grad_bucket: bool = False,
 ) -> nn.Module:
     """Turns ``module`` into one unit: its parameters (those no nested unit
     manages yet) move into a flat buffer sharded by ``planner`` for the
@@ -81,7 +82,9 @@ def matrix_fully_shard(
     here).  ``use_saved_tensor_hooks`` (default on, as in the reference) keeps
     autograd from pinning a unit's full buffer between forward and backward;
     ``full_param_buffer_pool`` (a ``FullParamBufferPool``) lets units of equal
-    size unshard into the same storage."""
+    size unshard into the same storage; ``use_zero_copy_grad_bucket`` (default
+    off, as in the reference) lets autograd write gradients straight into the
+    reduce-scatter workspace where the layout and dtypes allow it."""
     validate_mixed_precision_policy(mp_policy)
     if not isinstance(reshard_after_forward, bool):
         # an int asks for resharding to a smaller world after forward (matrix_fsdp/runtime/fsdp_unit.py:1705-1720)
@@ -104,6 +107,7 @@ def matrix_fully_shard(
         cast_forward_inputs=getattr(mp_policy, "cast_forward_inputs", True),
         use_saved_tensor_hooks=use_saved_tensor_hooks,
         full_param_buffer_pool=full_param_buffer_pool,
+        use_zero_copy_grad_bucket=use_zero_copy_grad_bucket,
     )
     if wrap_policy is not None:
         if shard_hints is not None:

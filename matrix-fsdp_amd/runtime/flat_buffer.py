@@ -383,6 +383,22 @@ class MatrixFlatBuffer:
         """Takes every parameter's ``.grad`` (flat_buffer.py:589-621).  The
         reduce-dtype cast is folded into the copy-in launch instead of being
         applied per grad."""
+        workspace = self.grad_bucket_input
+        if workspace is not None:
+            # zero-copy bucket: autograd has accumulated into views of the workspace, which then already is the
+            # reduce-scatter input (flat_buffer.py:447-486, 589-621).  A grad that was replaced instead of added to
+            # (create_graph, a hook) sends everything down the copy path.
+            offsets = self._packed_grad_offsets(compact=self.grad_bucket_input_is_compact)
+            base, size = workspace.data_ptr(), workspace.element_size()
+            in_place = all(
+                mp.param.grad is not None and mp.param.grad.dtype == workspace.dtype and mp.param.grad.data_ptr() == base + offsets[mp.fqn] * size
+                for mp in self.managed_params
+            )
+            self.grad_bucket_input = None
+            if in_place:
+                for mp in self.managed_params:
+                    mp.param.grad = None
+                return MatrixGradBucket((), self.plan.total_numel, self.shard_sizes, self.plan.rank_segments, packed_input=workspace, packed_input_is_compact=self.grad_bucket_input_is_compact)
         param_grads = []
         for mp in self.managed_params:
             grad = mp.param.grad
@@ -545,6 +561,8 @@ class MatrixFlatBuffer:
         one contiguous run of the workspace (flat_buffer.py:447-486)."""
         if self._param_compute_dtype() != self.local_shard.dtype or self.layout.max_shard_size == 0:
             return False
+        if self.reduce_dtype is not None and self.reduce_dtype != self.local_shard.dtype:
+            return False  # the workspace would have to be in the reduce dtype, which autograd cannot write into
         compact = self.is_whole_param_owner_layout()
         offsets = self._packed_grad_offsets(compact=compact)
         if any(off is None for off in offsets.values()):

@@ -137,6 +137,7 @@ class MatrixFSDPParamGroup:
         cast_forward_inputs: bool = True,
         use_saved_tensor_hooks: bool = True,
         full_param_buffer_pool=None,
+        use_zero_copy_grad_bucket: bool = False,
     ) -> None:
         if world_size < 1 or not 0 <= rank < world_size:
             raise ValueError(f"rank {rank} is outside a world of {world_size}.")
@@ -156,6 +157,7 @@ class MatrixFSDPParamGroup:
         self.cast_forward_inputs = cast_forward_inputs
         self.use_saved_tensor_hooks = use_saved_tensor_hooks
         self.full_param_buffer_pool = full_param_buffer_pool
+        self.use_zero_copy_grad_bucket = use_zero_copy_grad_bucket
         self._saved_tensor_contexts: list = []
         self.saved_full_param_views = 0
         self.managed_params: list[ManagedParam] = []
@@ -438,12 +440,17 @@ class MatrixFSDPParamGroup:
         if not self._backward_callback_queued:
             self._backward_callback_queued = True
             Variable._execution_engine.queue_callback(self._post_backward_callback)
-        if not self._in_backward and not self._finalized_after_backward:
+        entering = not self._in_backward and not self._finalized_after_backward
+        if entering:
             self._in_backward = True  # until finalize_backward
             self._stash_local_grads()
         if self.lifecycle_state != FSDPLifecycleState.UNSHARDED and not self._finalized_after_backward:
             self._record("pre_backward")
             self.unshard("pre_backward")
+        if entering and self.use_zero_copy_grad_bucket and self.flat_buffer.prepare_grad_bucket():
+            # the parameters are full again, so full-shaped views of the workspace can stand in as their grads:
+            # autograd accumulates into the reduce-scatter input directly and no copy-in launch is needed
+            self._record("zero_copy_grad_bucket")
         return grad
 
     def _post_accumulate_grad(self, param: torch.Tensor) -> None:
@@ -468,8 +475,8 @@ class MatrixFSDPParamGroup:
         if fb is None or self._finalized_after_backward:
             return
         bucket = fb.collect_grad_bucket()
-        if bucket.param_grads:
-            missing = [mp for mp in self.managed_params if all(pg.managed_param is not mp for pg in bucket.param_grads)]
+        if bucket.has_grads:
+            missing = [mp for mp in self.managed_params if all(pg.managed_param is not mp for pg in bucket.param_grads)] if bucket.param_grads else []
             if missing:
                 # parameters without a gradient contribute zeros, as a reduce-scatter of an untouched workspace would
                 zeros = [(mp, torch.zeros(mp.numel, dtype=bucket.param_grads[0].grad.dtype, device=fb.device)) for mp in missing]

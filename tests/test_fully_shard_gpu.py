@@ -707,3 +707,55 @@ def test_full_param_buffer_pool_shares_one_buffer_between_equal_units():
         assert rel(unit.flat_buffer.local_shard, ref_layer.w.detach().view(-1)[: dim * dim // world]) < 2e-6
     stats = pool.stats()
     assert stats["allocations"] <= 2 and stats["reuses"] >= 3 * 2 * depth - 1, stats
+
+
+class SkippableTail(nn.Module):
+    def __init__(self) -> None:
+        super().__init__()
+        self.body = nn.Sequential(nn.Linear(32, 48), nn.GELU(), nn.Linear(48, 16))
+        self.tail = nn.Linear(16, 16)
+
+    def forward(self, x, use_tail: bool = True):
+        x = self.body(x)
+        return self.tail(x) if use_tail else x
+
+
+@pytest.mark.parametrize("world, rank, planner, applies", [(1, 0, None, True), (3, 1, "owner", True), (4, 2, fsdp2_chunk_plan, False)])
+def test_zero_copy_grad_bucket_through_the_lifecycle(world, rank, planner, applies):
+    """``use_zero_copy_grad_bucket``: autograd accumulates into views of the reduce-scatter workspace, the backward
+    has no copy-in launch, and the reduced shard equals the copy-in path's bit for bit -- also over two
+    accumulated backwards and with an unused parameter.  Per-parameter chunks scatter a parameter over the
+    workspace's rows, so there the bucket declines and the copy-in path runs (test/fsdp/test_flat_buffer.py:1049-1063)."""
+    from matrix_fsdp_amd import matrix_fully_shard
+
+    shards = {}
+    for zero_copy in (False, True):
+        torch.manual_seed(7)
+        model = SkippableTail().to(DEV)
+        kwargs = {}
+        if planner == "owner":
+            kwargs["planner"] = lambda mps, w: whole_param_owner_plan(mps, w, [i % w for i in range(len(mps))])
+        elif planner is not None:
+            kwargs["planner"] = planner
+        matrix_fully_shard(model, world_size=world, rank=rank, use_zero_copy_grad_bucket=zero_copy, **kwargs)
+        unit = model._matrix_fsdp_param_group
+        gen = torch.Generator().manual_seed(8)
+        for micro in range(2):
+            x = torch.randn(8, 32, generator=gen).to(DEV)
+            out = model(x, use_tail=micro == 1)  # the first micro-batch leaves the last layer unused
+            out.square().mean().backward()
+            assert unit.lifecycle_state == FSDPLifecycleState.SHARDED and unit.flat_buffer.grad_bucket_input is None
+        assert ("zero_copy_grad_bucket" in unit.events) == (zero_copy and applies)
+        shards[zero_copy] = unit.flat_buffer.local_grad_shard.clone()
+        assert all(p.grad is None or p.grad.untyped_storage().data_ptr() == unit.flat_buffer.local_grad_shard.untyped_storage().data_ptr() for p in model.parameters())
+    assert torch.equal(shards[True], shards[False])
+
+
+def test_zero_copy_grad_bucket_declines_under_mixed_precision():
+    from matrix_fsdp_amd import matrix_fully_shard
+
+    model = nn.Linear(16, 16).to(DEV)
+    matrix_fully_shard(model, world_size=2, rank=0, use_zero_copy_grad_bucket=True, mp_policy=MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32))
+    model(torch.randn(4, 16, device=DEV)).float().square().mean().backward()
+    unit = model._matrix_fsdp_param_group
+    assert "zero_copy_grad_bucket" not in unit.events and unit.flat_buffer.local_grad_shard.dtype == torch.float32
