@@ -255,14 +255,14 @@ def main() -> int:
             for p, g, buf in mats:
                 F.muon_step(p, g, buf, workspace=ws, **kw)
 
-        med, _ = time_launches(torch, muon_all, 10, 3)
+        med, _ = time_launches(torch, muon_all, 20, 5)
         flops = 0
         per_matrix = {}
         for (p, g, buf), shape in zip(mats, MUON_HIDDEN4096_SHAPES):
             m, n = min(shape), max(shape)
             fl = 5 * (4 * m * m * n + 2 * m**3)
             flops += fl
-            t, _ = time_launches(torch, lambda: F.muon_step(p, g, buf, workspace=ws, **kw), 10, 2)
+            t, _ = time_launches(torch, lambda: F.muon_step(p, g, buf, workspace=ws, **kw), 20, 5)
             per_matrix[f"{shape[0]}x{shape[1]}"] = {"ms": round(t, 4), "TFLOPs": round(fl / (t * 1e-3) / 1e12, 1)}
         tflops = flops / (med * 1e-3) / 1e12
         legs["muon_hidden4096"] = {
