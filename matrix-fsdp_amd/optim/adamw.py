@@ -4,10 +4,11 @@ Hyper-parameters, parameter-group keys and state keys (``step``, ``exp_avg``,
 ``exp_avg_sq``) are those of ``torch.optim.AdamW`` (``amsgrad`` and ``maximize`` included), the optimizer the reference
 builds for everything Muon does not take (matrix_fsdp/optim/wrapper.py:431-439);
 the arithmetic is the single-tensor path of torch/optim/adam.py:347-547.  When
-the parameters are views of one flat shard, their grads views of one local
-grad shard and their moments views of flat state buffers
-(``initialize_flat_adamw_state``), neighbouring parameters are merged and the
-whole shard is updated by a single launch.
+the parameters are views of one flat shard and their grads views of one local
+grad shard, neighbouring parameters are merged and the run is updated by a
+single launch: the moments this optimizer creates for such a run are laid out
+back to back as well (``initialize_flat_adamw_state`` does the same for a whole
+flat buffer up front and keeps the buffers addressable).
 """
 from __future__ import annotations
 
@@ -45,15 +46,27 @@ class FusedAdamW(Optimizer):
         defaults = {"lr": lr, "betas": betas, "eps": eps, "weight_decay": weight_decay, "amsgrad": bool(amsgrad), "maximize": bool(maximize)}
         super().__init__(params, defaults)
 
-    def _init_state(self, p: Tensor, amsgrad: bool) -> dict:
-        state = self.state[p]
-        if len(state) == 0:
-            state["step"] = torch.tensor(0.0, dtype=torch.float32)
-            state["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-            state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-            if amsgrad:
-                state["max_exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
-        return state
+    def _init_states(self, params: list[Tensor], amsgrad: bool) -> None:
+        """First step: parameters that follow each other in memory (views of one local shard) get moments that
+        follow each other too, so that the run can be updated by one launch.  Every parameter still has its own
+        ``exp_avg`` / ``exp_avg_sq`` tensors of its own shape."""
+        fresh = sorted((p for p in params if len(self.state[p]) == 0), key=lambda p: p.data_ptr())
+        names = ("exp_avg", "exp_avg_sq") + (("max_exp_avg_sq",) if amsgrad else ())
+        start = 0
+        while start < len(fresh):
+            end = start + 1
+            while end < len(fresh) and _follows(fresh[end - 1].data, fresh[end].data):
+                end += 1
+            run = fresh[start:end]
+            flats = {name: torch.zeros(sum(p.numel() for p in run), dtype=run[0].dtype, device=run[0].device) for name in names}
+            cursor = 0
+            for p in run:
+                state = self.state[p]
+                state["step"] = torch.tensor(0.0, dtype=torch.float32)
+                for name in names:
+                    state[name] = flats[name][cursor : cursor + p.numel()].view(p.shape)
+                cursor += p.numel()
+            start = end
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -64,14 +77,17 @@ class FusedAdamW(Optimizer):
         for group in self.param_groups:
             amsgrad = bool(group.get("amsgrad", False))
             entries = []
-            for p in group["params"]:
-                if p.grad is None or p.numel() == 0:
-                    continue
+            active = [p for p in group["params"] if p.grad is not None and p.numel() > 0]
+            for p in active:
                 if p.grad.is_sparse:
                     raise RuntimeError("AdamW does not support sparse gradients")
                 if p.dtype != torch.float32:
                     raise RuntimeError(f"FusedAdamW updates float32 parameters, got {p.dtype}")
-                state = self._init_state(p, amsgrad)
+            self._init_states(active, amsgrad)
+            for p in active:
+                state = self.state[p]
+                if amsgrad and "max_exp_avg_sq" not in state:  # amsgrad switched on after the first step
+                    state["max_exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 state["step"] += 1
                 tensors = [p.data, p.grad.contiguous(), state["exp_avg"], state["exp_avg_sq"]]
                 if amsgrad:

@@ -93,6 +93,56 @@ def test_fused_adamw_merges_flat_views_into_one_launch_and_matches_torch():
         FusedAdamW(ours, betas=(1.0, 0.9))
 
 
+def test_fused_adamw_lays_out_its_own_moments_for_contiguous_parameters(monkeypatch):
+    """Without any flat-state set-up: parameters that are views of one shard get back-to-back moments at the first
+    step, so the whole run is one launch per step; a parameter elsewhere in memory keeps its own launch; amsgrad
+    adds its running maximum to the same layout.  Results as ``torch.optim.AdamW``."""
+    from matrix_fsdp_amd.optim import adamw as adamw_module
+
+    gen = torch.Generator().manual_seed(3)
+    sizes = [(6, 4), (5,), (2, 8)]
+    total = sum(torch.Size(s).numel() for s in sizes)
+    flat_p = (torch.randn(total, generator=gen) * 0.02).to(DEV)
+    ours, refs, off = [], [], 0
+    for s in sizes + [(9,)]:
+        n = torch.Size(s).numel()
+        p = nn.Parameter(flat_p[off : off + n].view(s)) if s != (9,) else nn.Parameter((torch.randn(9, generator=gen) * 0.02).to(DEV))
+        ours.append(p)
+        refs.append(nn.Parameter(p.detach().cpu().clone()))
+        off += n
+    kw = dict(lr=1e-3, betas=(0.9, 0.99), eps=1e-8, weight_decay=0.05, amsgrad=True)
+    opt, opt_ref = FusedAdamW(ours, **kw), torch.optim.AdamW(refs, foreach=False, **kw)
+    launches = []
+    real = adamw_module.F.adamw_step
+    monkeypatch.setattr(adamw_module.F, "adamw_step", lambda *a, **k: (launches.append(a[0].numel()), real(*a, **k))[1])
+    for step in range(3):
+        flat_g = (torch.randn(total + 9, generator=gen) * 1e-3).to(DEV)  # one grad shard, as after a backward
+        off = 0
+        for p, r in zip(ours, refs):
+            p.grad = flat_g[off : off + p.numel()].view(p.shape)
+            r.grad = p.grad.cpu().clone()
+            off += p.numel()
+        launches.clear()
+        opt.step()
+        opt_ref.step()
+        assert sorted(launches) == [9, total], launches
+    first, second = opt.state[ours[0]], opt.state[ours[1]]
+    for name in ("exp_avg", "exp_avg_sq", "max_exp_avg_sq"):
+        assert second[name].data_ptr() == first[name].data_ptr() + ours[0].numel() * 4 and first[name].shape == ours[0].shape
+    for p, r in zip(ours, refs):
+        assert torch.allclose(p.detach().cpu(), r.detach(), rtol=1e-6, atol=1e-8)
+        for name in ("exp_avg", "exp_avg_sq", "max_exp_avg_sq"):
+            assert torch.allclose(opt.state[p][name].cpu(), opt_ref.state[r][name], rtol=1e-5, atol=1e-12), name
+    # a state dict loaded back gives every parameter its own tensors again: still correct, one launch each
+    opt.load_state_dict(opt.state_dict())
+    launches.clear()
+    opt.step()
+    opt_ref.step()
+    assert len(launches) in (2, 4)
+    for p, r in zip(ours, refs):
+        assert torch.allclose(p.detach().cpu(), r.detach(), rtol=1e-6, atol=1e-8)
+
+
 def build_owner_buffers():
     """Two units; every matrix whole on its owner, rank 0 owning every second parameter."""
     gen = torch.Generator().manual_seed(2)
