@@ -494,9 +494,12 @@ class MatrixFlatBuffer:
         else:
             packed = torch.empty(self.layout.padded_numel, dtype=reduce_dtype, device=self.device)
             fill_reduce_scatter_input(bucket, packed, backend=backend, cache=self._copy_in_cache)
-        chunk = torch.empty(self.shard_sizes[self.rank], dtype=packed.dtype, device=self.device)
         offset = self.plan.rank_packed_offset(self.rank) if compact else self.rank * self.layout.max_shard_size
-        native.copy_range(packed, chunk, offset)
+        if offset == 0 and packed.numel() == self.shard_sizes[self.rank]:
+            chunk = packed  # a world of one: the workspace is the shard, no second pass over the gradients
+        else:
+            chunk = torch.empty(self.shard_sizes[self.rank], dtype=packed.dtype, device=self.device)
+            native.copy_range(packed, chunk, offset)
         reduced = self._maybe_to_local_dtype(chunk)
         if accumulate and self.local_grad_shard is not None:
             self.accumulate_local_grad_shard(reduced)
