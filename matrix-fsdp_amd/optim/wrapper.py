@@ -330,7 +330,7 @@ class PreparedMatrixOptimizer:
     def _zero_grad(self, *args: Any, **kwargs: Any) -> None:
         self._refuse_inside_no_sync("optimizer.zero_grad")
         for unit in self._fsdp_param_groups:
-            if unit._in_backward:
+            if unit.has_pending_backward_reduce:
                 unit.finalize_backward()
         self._original_zero_grad(*args, **kwargs)
         for unit in self._fsdp_param_groups:

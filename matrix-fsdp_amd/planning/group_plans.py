@@ -19,6 +19,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 from itertools import accumulate
+from types import SimpleNamespace
 from typing import Callable, Sequence
 
 from ..core.layout import LayoutSegment, MatrixGroupLayout, ShardPlan
@@ -409,9 +410,5 @@ def rotate_layout_ranks(layout: MatrixGroupLayout, rank_offset: int) -> MatrixGr
         return layout
     shift = rank_offset % world
     rolled = tuple(layout.rank_segments[(rank - shift) % world] for rank in range(world))
-
-    class _Span:  # what from_shard_plan needs to know of a parameter
-        def __init__(self, p):
-            self.fqn, self.offset, self.end = p.fqn, p.global_start, p.global_end
-
-    return MatrixGroupLayout.from_shard_plan(ShardPlan.from_rank_segments(layout.total_numel, rolled), [_Span(p) for p in layout.params])
+    spans = [SimpleNamespace(fqn=p.fqn, offset=p.global_start, end=p.global_end) for p in layout.params]
+    return MatrixGroupLayout.from_shard_plan(ShardPlan.from_rank_segments(layout.total_numel, rolled), spans)

@@ -275,6 +275,11 @@ class MatrixFSDPParamGroup:
     def no_sync(self) -> MatrixFSDPNoSync:
         return MatrixFSDPNoSync([self])
 
+    @property
+    def has_pending_backward_reduce(self) -> bool:
+        """A backward has started on this unit and its gradients have not been reduced into the local shard yet."""
+        return self._in_backward
+
     def is_no_sync_active(self) -> bool:
         return self._no_sync_depth > 0
 
