@@ -31,6 +31,26 @@ _MUON_OPTIMIZER_POLICIES = {"mixed_muon_adamw", "muon_adamw", "muon_shard_aware"
 _NOOP_OPTIMIZER_POLICIES = {"default", "none", "adamw", "sgd"}
 
 
+# arguments of the reference's matrix_fully_shard (matrix_fsdp/api.py:266-300) that choose collectives, their
+# scheduling or tracing: nothing for them to steer without a process group
+_SINGLE_DEVICE_NOOPS = frozenset(
+    {
+        "dp_mesh_dims",
+        "dp_shard_mesh_dim",
+        "dp_replicate_mesh_dim",
+        "forward_prefetch",
+        "backward_prefetch",
+        "param_gather_strategy",
+        "matrix_collective_backend",
+        "grad_reduce_strategy",
+        "backward_reduce_strategy",
+        "runtime_layout_policy",
+        "runtime_trace_enabled",
+        "shrink_full_param_storage_after_backward",
+    }
+)
+
+
 @dataclass(frozen=True)
 class MixedPrecisionPolicy:
     """Field-compatible with ``torch.distributed.fsdp.MixedPrecisionPolicy``, which is accepted as well."""
@@ -67,6 +87,11 @@ def matrix_fully_shard(
     use_saved_tensor_hooks: bool = True,
     full_param_buffer_pool=None,
     use_zero_copy_grad_bucket: bool = False,
+    mesh=None,
+    group_planner: Callable[[list[ManagedParam], int], ShardPlan] | None = None,
+    offload_policy=None,
+    finalize_after_backward: bool = True,
+    **single_device_noops,
 ) -> nn.Module:
     """Turns ``module`` into one unit: its parameters (those no nested unit
     manages yet) move into a flat buffer sharded by ``planner`` for the
@@ -84,7 +109,26 @@ def matrix_fully_shard(
     ``full_param_buffer_pool`` (a ``FullParamBufferPool``) lets units of equal
     size unshard into the same storage; ``use_zero_copy_grad_bucket`` (default
     off, as in the reference) lets autograd write gradients straight into the
-    reduce-scatter workspace where the layout and dtypes allow it."""
+    reduce-scatter workspace where the layout and dtypes allow it.
+
+    Of the reference's further arguments, ``group_planner`` is ``planner``
+    under its other name; ``mesh`` (one rank at most), ``offload_policy`` (no
+    offload) and ``finalize_after_backward`` (``True``) are taken in their
+    neutral values; the switches that only choose collectives or the order in
+    which they are issued (``_SINGLE_DEVICE_NOOPS``) are accepted and have no
+    effect on one device.  Anything else is a ``TypeError``."""
+    unknown = set(single_device_noops) - _SINGLE_DEVICE_NOOPS
+    if unknown:
+        raise TypeError(f"matrix_fully_shard() got unexpected keyword arguments: {', '.join(sorted(unknown))}.")
+    _refuse_multi_device_arguments(mesh, offload_policy, single_device_noops.get("dp_mesh_dims"))
+    if any(single_device_noops.get(name) is not None for name in ("dp_shard_mesh_dim", "dp_replicate_mesh_dim")):
+        raise NotImplementedError("dp_shard_mesh_dim / dp_replicate_mesh_dim select dimensions of a multi-rank mesh, which does not exist here.")
+    if not finalize_after_backward:
+        raise NotImplementedError("finalize_after_backward=False leaves the reduce to the caller; units here always finalise at the end of the backward.")
+    if group_planner is not None:
+        if planner is not None:
+            raise ValueError("Pass either planner or group_planner, not both.")
+        planner = group_planner
     validate_mixed_precision_policy(mp_policy)
     if not isinstance(reshard_after_forward, bool):
         # an int asks for resharding to a smaller world after forward (matrix_fsdp/runtime/fsdp_unit.py:1705-1720)

@@ -272,6 +272,20 @@ def test_fully_shard_host_rules():
         fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: Replicate())
     with pytest.raises(NotImplementedError, match="supports only Shard\\(0\\)"):
         fully_shard(torch.nn.Linear(2, 2), shard_placement_fn=lambda p: Shard(1))
+    # matrix_fully_shard: switches that only steer collectives are accepted, anything unknown is not
+    from matrix_fsdp_amd import matrix_fully_shard as mfs
+    from matrix_fsdp_amd.core.plans import fsdp2_chunk_plan
+
+    with pytest.raises(TypeError, match="unexpected keyword arguments: prefetch_depth"):
+        mfs(torch.nn.Linear(2, 2), forward_prefetch=True, prefetch_depth=2)
+    with pytest.raises(NotImplementedError, match="finalize_after_backward=False"):
+        mfs(torch.nn.Linear(2, 2), finalize_after_backward=False)
+    with pytest.raises(ValueError, match="either planner or group_planner"):
+        mfs(torch.nn.Linear(2, 2), planner=fsdp2_chunk_plan, group_planner=fsdp2_chunk_plan)
+    with pytest.raises(NotImplementedError, match="dp_shard_mesh_dim"):
+        mfs(torch.nn.Linear(2, 2), dp_shard_mesh_dim=0)
+    with pytest.raises(RuntimeError, match="HIP device"):  # every argument accepted: stops only at the CPU module
+        mfs(torch.nn.Linear(2, 2), forward_prefetch=True, backward_prefetch=False, matrix_collective_backend="custom", group_planner=fsdp2_chunk_plan, world_size=2)
     # wrap policies decide before anything touches the device
     from matrix_fsdp_amd import matrix_fully_shard
     from matrix_fsdp_amd.policy import module_type_policy
