@@ -14,12 +14,14 @@ from __future__ import annotations
 
 import torch
 from torch import Tensor
-from torch.optim.optimizer import Optimizer
 
 from . import functional as F
 
 
-class FusedAdamW(Optimizer):
+class FusedAdamW(torch.optim.AdamW):
+    """A ``torch.optim.AdamW`` (same constructor checks, defaults, parameter-group and state keys, so state dicts
+    are interchangeable) whose ``step`` runs on the HIP kernel."""
+
     def __init__(
         self,
         params,
@@ -33,18 +35,7 @@ class FusedAdamW(Optimizer):
     ) -> None:
         if isinstance(lr, Tensor):
             raise ValueError("FusedAdamW takes a float lr")
-        if not 0.0 <= lr:
-            raise ValueError(f"Invalid learning rate: {lr}")
-        if not 0.0 <= eps:
-            raise ValueError(f"Invalid epsilon value: {eps}")
-        if not 0.0 <= betas[0] < 1.0:
-            raise ValueError(f"Invalid beta parameter at index 0: {betas[0]}")
-        if not 0.0 <= betas[1] < 1.0:
-            raise ValueError(f"Invalid beta parameter at index 1: {betas[1]}")
-        if not 0.0 <= weight_decay:
-            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
-        defaults = {"lr": lr, "betas": betas, "eps": eps, "weight_decay": weight_decay, "amsgrad": bool(amsgrad), "maximize": bool(maximize)}
-        super().__init__(params, defaults)
+        super().__init__(params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=bool(amsgrad), maximize=bool(maximize), foreach=False)
 
     def _init_states(self, params: list[Tensor], amsgrad: bool) -> None:
         """First step: parameters that follow each other in memory (views of one local shard) get moments that

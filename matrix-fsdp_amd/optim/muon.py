@@ -10,8 +10,6 @@ matrix through ``mfsdp_muon_step``; nothing falls back to torch arithmetic.
 from __future__ import annotations
 
 import torch
-from torch import Tensor
-from torch.optim.optimizer import Optimizer
 
 from . import functional as F
 
@@ -20,7 +18,9 @@ DEFAULT_A, DEFAULT_B, DEFAULT_C = F.NS_COEFFICIENTS
 DEFAULT_NS_STEPS = F.NS_STEPS
 
 
-class Muon(Optimizer):
+class Muon(torch.optim.Muon):
+    """A ``torch.optim.Muon`` (same constructor checks, defaults and state) whose ``step`` runs on the HIP kernels."""
+
     def __init__(
         self,
         params,
@@ -33,31 +33,10 @@ class Muon(Optimizer):
         ns_steps: int = DEFAULT_NS_STEPS,
         adjust_lr_fn: str | None = None,
     ) -> None:
-        if isinstance(lr, Tensor) and lr.numel() != 1:
-            raise ValueError("Tensor lr must be 1-element")
-        if not 0.0 <= lr:
-            raise ValueError(f"Learning rate should be >= 0 but is: {lr}")
-        if not 0.0 <= momentum:
-            raise ValueError(f"momentum should be >= 0 but is: {momentum}")
-        if not 0.0 <= weight_decay:
-            raise ValueError(f"weight decay should be >= 0 but is: {weight_decay}")
-        if adjust_lr_fn is not None and adjust_lr_fn not in ("original", "match_rms_adamw"):
-            raise ValueError(f"Adjust learning rate function {adjust_lr_fn} is not supported")
-        defaults = {
-            "lr": lr,
-            "weight_decay": weight_decay,
-            "momentum": momentum,
-            "nesterov": nesterov,
-            "ns_coefficients": ns_coefficients,
-            "eps": eps,
-            "ns_steps": ns_steps,
-            "adjust_lr_fn": adjust_lr_fn,
-        }
-        super().__init__(params, defaults)
-        for group in self.param_groups:
-            for p in group["params"]:
-                if p.ndim != 2:
-                    raise ValueError(f"Muon only supports 2D parameters whereas we found a parameter with size: {p.size()}")
+        super().__init__(
+            params, lr=lr, weight_decay=weight_decay, momentum=momentum, nesterov=nesterov, ns_coefficients=ns_coefficients,
+            eps=eps, ns_steps=ns_steps, adjust_lr_fn=adjust_lr_fn,
+        )
         self._workspace: F.MuonWorkspace | None = None
 
     @torch.no_grad()

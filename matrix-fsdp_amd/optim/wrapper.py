@@ -457,6 +457,27 @@ def _local_params(module_or_units) -> list[nn.Parameter]:
     return params
 
 
+_SCHEDULER_KWARG_NAMES = frozenset(
+    {
+        "max_unsharded_prefetch_units",
+        "max_forward_prefetch_units",
+        "max_backward_prefetch_units",
+        "backward_prefetch_timing",
+        "prefetch_policy",
+        "max_cached_full_param_buffers_per_key",
+        "max_cached_elastic_workspaces_per_key",
+        "max_active_full_param_buffers",
+        "max_active_full_param_numel",
+        "max_active_full_param_memory_mb",
+        "max_pending_backward_reduces",
+        "owner_backward_prefetch_with_pending_reduce",
+        "trim_cuda_cache",
+        "cuda_cache_trim_threshold_mb",
+        "scheduler_config",
+    }
+)
+
+
 def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig = "adamw", **kwargs: Any):
     """``'adamw'`` / ``'sgd'`` / ``'muon'`` / ``'mixed_muon_adamw'`` (aliases
     ``'muon_adamw'``, ``'mixed'``) over the local parameters of the given
@@ -473,10 +494,16 @@ def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig 
     optimizer_kwargs.update(kwargs)
     default_matrix_optimizer = optimizer_kwargs.pop("default_matrix_optimizer", default_matrix_optimizer)
     default_other_optimizer = optimizer_kwargs.pop("default_other_optimizer", default_other_optimizer)
+    # the reference routes these to its prefetch scheduler (matrix_fsdp/optim/wrapper.py:32-51, 939-942); one device
+    # has nothing to schedule, so they are taken and dropped -- all but flat_adamw_state, which is a layout choice
+    flat_adamw_state = bool(optimizer_kwargs.pop("flat_adamw_state", False))
+    for name in _SCHEDULER_KWARG_NAMES:
+        optimizer_kwargs.pop(name, None)
     kind = kind.lower()
     if kind in ("mixed_muon_adamw", "muon_adamw", "mixed"):
         return make_mixed_muon_adamw_optimizer(
-            module_or_units, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer, **optimizer_kwargs
+            module_or_units, default_matrix_optimizer=default_matrix_optimizer, default_other_optimizer=default_other_optimizer,
+            flat_adamw_state=flat_adamw_state, **optimizer_kwargs
         )
     params = _local_params(module_or_units)
     with _without_auto_prepare():  # prepared below, for the units of module_or_units
@@ -491,7 +518,7 @@ def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig 
     if built is not None:
         units = units_of(module_or_units)
         if units:
-            prepare_matrix_optimizer(built, units)
+            prepare_matrix_optimizer(built, units, flat_adamw_state=flat_adamw_state and kind == "adamw")
         return built
     raise ValueError(f"optimizer must be one of 'adamw', 'sgd', 'muon', or 'mixed_muon_adamw', got {kind!r}.")
 

@@ -231,3 +231,33 @@ def test_muon_hint_on_partial_parameter_is_rejected():
     with pytest.raises(ValueError, match="optimizer must be one of"):
         configure_optimizer([fb], "lion")
     assert isinstance(configure_optimizer([fb], "adamw", lr=1e-3), FusedAdamW)
+
+
+def test_hip_optimizers_are_torch_optimizers_of_the_same_kind():
+    """``configure_optimizer(..., "adamw")`` is a ``torch.optim.AdamW`` in the reference
+    (test/fsdp/test_matrix_fsdp_e2e.py:1911-1912); the HIP optimizers subclass torch's, share their constructor
+    checks and their state-dict layout, and take the reference's scheduler keywords without effect."""
+    from matrix_fsdp_amd import configure_optimizer, fully_shard
+    from matrix_fsdp_amd.optim.muon import Muon
+
+    model = nn.Sequential(nn.Linear(8, 8), nn.Linear(8, 4)).to(DEV)
+    fully_shard(model)
+    opt = configure_optimizer(model, "adamw", lr=1e-2, max_forward_prefetch_units=2, prefetch_policy="static", trim_cuda_cache=True)
+    assert isinstance(opt, torch.optim.AdamW) and isinstance(opt, FusedAdamW)
+    twin = torch.optim.AdamW([nn.Parameter(p.detach().clone()) for p in model.parameters()], lr=1e-2, foreach=False)
+    assert set(opt.param_groups[0]) == set(twin.param_groups[0])
+    model(torch.randn(4, 8, device=DEV)).sum().backward()
+    opt.step()
+    twin.load_state_dict(opt.state_dict())  # interchangeable state dicts
+    assert float(twin.state[twin.param_groups[0]["params"][0]]["step"]) == 1.0
+    muon = Muon([p for p in model.parameters() if p.ndim == 2], lr=1e-2)
+    assert isinstance(muon, torch.optim.Muon)
+    with pytest.raises(ValueError, match="only supports 2D"):
+        Muon(list(model.parameters()))
+    with pytest.raises(ValueError, match="Learning rate should be >= 0"):
+        Muon([p for p in model.parameters() if p.ndim == 2], lr=-1.0)
+    flat = configure_optimizer(model, "adamw", lr=1e-2, flat_adamw_state=True)
+    model(torch.randn(4, 8, device=DEV)).sum().backward()
+    flat.step()
+    first, second = (flat.state[p]["exp_avg"] for p in list(model.parameters())[:2])
+    assert second.data_ptr() == first.data_ptr() + first.numel() * 4
