@@ -386,3 +386,35 @@ def test_full_param_buffer_pool_bookkeeping():
 
     with pytest.raises(ValueError, match="needs use_saved_tensor_hooks"):
         MatrixFSDPParamGroup(torch.nn.Linear(2, 2), full_param_buffer_pool=FullParamBufferPool(max_cached_per_key=1), use_saved_tensor_hooks=False)
+
+
+def test_public_names_of_the_reference_that_this_build_provides():
+    """The reference's top-level names for the path, its metadata, the lifecycle shell, the planners and the
+    checkpoint format resolve on this package too (what is left out needs a process group: meshes, DTensor
+    placements, collectives, the prefetch scheduler, the auto planner with its cost model)."""
+    import matrix_fsdp_amd as m
+
+    assert all(hasattr(m, name) for name in m.__all__)
+    provided = """
+        LayoutSegment ShardPlan MatrixGroupLayout ParamLayout ParamSegment RankLayout ManagedParam ManagedParamRegistry
+        ParamShardHint ParamRuntimeKind MatrixShard PlacementCompatibility MatrixShardedState MixedPrecisionPolicy
+        StaticParamBufferLayout ElasticParamBufferLayout ElasticCommunicationPlan ElasticRankChunk FullParamBufferPool
+        FSDPLifecycleState MatrixFSDPParamGroup MatrixFSDPNoSync WrapPolicy
+        fully_shard matrix_fully_shard configure_optimizer configure_matrix_optimizer prepare_matrix_optimizer
+        install_matrix_optimizer_auto_prepare PreparedMatrixOptimizer MatrixFSDPOptimizer MixedMuonAdamWOptimizer
+        MatrixOptimizerConfig MatrixOptimizerParamGroupSummary ClassifiedMatrixOptimizerParams classify_matrix_optimizer_params
+        make_mixed_muon_adamw_optimizer collect_param_groups DEFAULT_MUON_ADJUST_LR_FN
+        MatrixFSDPOptimizerStateManager LocalOptimizerStateTensor OptimizerStateSummary
+        build_shard_hints moe_expert_owner_rule fsdp2_chunk_plan hinted_ordered_group_plan ordered_matrix_owner_tail_plan
+        load_balanced_matrix_owner_tail_plan load_balanced_matrix_owner_tail_group_plans expert_owner_tail_plan
+        explain_matrix_shard_compatibility is_matrix_shard_compatible_plan matrix_shard_from_plan matrix_shard_from_layout
+        shard_sizes_to_matrix_local_units matrix_shard_metadata matrix_sharded_state_metadata
+        explain_runtime_layout_compatibility validate_runtime_layout RuntimeLayoutCompatibility
+        rank_segments_are_rank_contiguous_chunks clear_global_full_param_buffer_pool
+        module_type_policy size_based_policy or_policy and_policy not_policy
+        matrix_state_dict load_matrix_state_dict save_matrix_dcp load_matrix_dcp load_matrix_dcp_full_state
+        get_state_dict set_state_dict get_model_state_dict set_model_state_dict get_optimizer_state_dict set_optimizer_state_dict
+        patch_model_state_dict patch_optimizer_state_dict matrix_get_state_dict matrix_set_state_dict
+    """.split()
+    missing = [name for name in provided if not hasattr(m, name)]
+    assert not missing, missing
