@@ -24,6 +24,7 @@ namespace {
 constexpr int kMaxSources = 128;  // pointer table passed by value in the kernel arguments
 constexpr int kWaveSize = 64;
 constexpr int kBlockThreads = 256;
+constexpr int64_t kMaxGrid = (int64_t{1} << 31) - 1;  // grid-stride loops keep a capped grid correct
 constexpr int kWavesPerBlock = kBlockThreads / kWaveSize;
 constexpr uint32_t kMaxGroupsPerRun = 0x7fffffffu;  // reciprocal division is exact below 2^31
 
@@ -209,7 +210,6 @@ segment_program_kernel(SourceTable srcs, char* __restrict__ dst, const DevRun* _
 
 struct Tuning {
   int blocks_per_cu = 2;        // persistent grid of the segment kernel: 2 workgroups (8 waves) per CU measured best
-  int linear_blocks_per_cu = 16;  // contiguous range copies / casts want more workgroups in flight
   int nontemporal = 1;
   int unroll = 4;
   // elements per lane when converting: 4 keeps the wider side at one 16-byte access per lane, so that every wave-level
@@ -652,8 +652,9 @@ int launch_linear(const char* src, char* dst, int64_t n_groups, hipStream_t stre
   constexpr int U = 4;
   const int64_t span = static_cast<int64_t>(kBlockThreads) * U;
   const int64_t want = (n_groups + span - 1) / span;
-  const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.linear_blocks_per_cu);
-  const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, cap))));
+  // one workgroup per block of the tensor, not a persistent grid: workgroups are dispatched in order, so those in
+  // flight sweep neighbouring addresses (bf16 -> fp32 of 202 M elements 5.83 against 5.65 TB/s with 16 per CU)
+  const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, kMaxGrid))));
   if (g_tuning.nontemporal)
     hipLaunchKernelGGL((linear_kernel<SRC_B, DST_B, U, true, HALF>), grid, dim3(kBlockThreads), 0, stream, src, dst, n_groups);
   else
@@ -772,8 +773,8 @@ extern "C" int mfsdp_accumulate(void* dst, const void* src, int64_t numel, int d
   const int64_t tail_first = n_vec * per_vec, tail = numel - tail_first;
   const int64_t work = std::max(n_vec, tail);
   const int64_t want = (work + kBlockThreads - 1) / kBlockThreads;
-  const int64_t cap = static_cast<int64_t>(device_cu_count()) * std::max(1, g_tuning.linear_blocks_per_cu);
-  const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, cap))));
+  // one workgroup per block, as launch_linear: 6.27 against 4.78 TB/s with 16 persistent workgroups per CU (fp32, 202 M elements)
+  const dim3 grid(static_cast<uint32_t>(std::max<int64_t>(1, std::min(want, kMaxGrid))));
   char* d = static_cast<char*>(dst);
   const char* s = static_cast<const char*>(src);
   if (dtype == MFSDP_F32) hipLaunchKernelGGL((accumulate_kernel<0>), grid, dim3(kBlockThreads), 0, as_stream(stream), d, s, n_vec, tail_first, tail);
