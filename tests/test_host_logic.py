@@ -418,3 +418,22 @@ def test_public_names_of_the_reference_that_this_build_provides():
     """.split()
     missing = [name for name in provided if not hasattr(m, name)]
     assert not missing, missing
+
+
+def test_bench_refuses_more_than_one_gpu_and_the_product_has_no_cpu_path():
+    """``bench.py --gpus N`` with N above 1 exits with a message before touching a device; the flat buffer refuses
+    host tensors instead of falling back to host copies."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    done = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert done.returncode != 0 and "ONE GPU" in (done.stdout + done.stderr) and not done.stdout.strip().startswith("{")
+    from matrix_fsdp_amd.core.managed_param import managed_params_from_module
+    from matrix_fsdp_amd.core.plans import contiguous_even_plan
+    from matrix_fsdp_amd.runtime.flat_buffer import MatrixFlatBuffer
+
+    params = list(managed_params_from_module(torch.nn.Linear(4, 4)))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        MatrixFlatBuffer(params, contiguous_even_plan(params[-1].end, 2), rank=0)
