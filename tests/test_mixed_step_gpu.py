@@ -1,13 +1,17 @@
 """The mixed optimizer step of the whole-parameter owner layout, end to end on reduced shapes: gradient copy-in for
 the owner layout, Muon on the matrices rank 0 owns, fused AdamW on its fp32 tail shard, and pack / unpack of the
 rank-major flat buffers -- every stage against the CPU oracle (copies bit-exact, Muon within the stated tolerance),
-plus the full-size Newton-Schulz shapes of the hidden4096 model against the oracle."""
+plus, at full size, every matrix shape of the hidden4096 and hidden5120 models (Newton-Schulz output and parameter
+delta) and one hidden5120 layer buffer with the AdamW tail shard."""
+import json
+import os
+
 import pytest
 import torch
 
 from matrix_fsdp_amd.kernels.segment_program import compact_owner_program, pack_program, unpack_program
 from matrix_fsdp_amd.optim import functional as F
-from matrix_fsdp_amd.workloads import ParamSpec, Workload, normal_flat, transformer_layer_shapes
+from matrix_fsdp_amd.workloads import HIDDEN5120, HIDDEN5120_TAIL_NUMEL, ParamSpec, Workload, normal_flat, transformer_layer_shapes
 from oracle import copy_oracle as CO
 from oracle import optim_oracle as OO
 from tests.test_copy_gpu import assert_same_bits
@@ -91,10 +95,27 @@ def test_rank0_mixed_update_over_all_layers():
         assert max_err_over_scale(have, want) < 1e-6
 
 
-@pytest.mark.parametrize("shape", [(4096, 4096), (4096, 11008)])
+# Every matrix shape of the two measured models, in the orientation the model holds it: the hidden4096 layer
+# (m = 4096: 128 x 128 triangle tiles for the symmetric products) and the hidden5120 layer (m = 5120: the 256 x 256
+# triangle tile with mirrored store; tall inputs run on the transposed orientation and the last step writes only the
+# transposed output; n = 13824 leaves K-split remainder tiles for the fix-up kernel).
+FULL_SIZE_SHAPES = [
+    (4096, 4096), (12288, 4096), (11008, 4096), (4096, 11008),
+    (5120, 5120), (15360, 5120), (13824, 5120), (5120, 13824),
+]
+
+
+def _report(record: dict) -> None:
+    """Measured distances are appended, one JSON object per line, to the file MFSDP_PARITY_REPORT names (when set)."""
+    path = os.environ.get("MFSDP_PARITY_REPORT")
+    if path:
+        with open(path, "a") as f:
+            f.write(json.dumps(record) + "\n")
+
+
+@pytest.mark.parametrize("shape", FULL_SIZE_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
 def test_newton_schulz_full_size_against_oracle(shape):
-    """The bench shapes themselves (the wide one in its transposed, cheaper-for-the-CPU orientation is the same
-    arithmetic: both sides transpose tall inputs first).
+    """The bench shapes themselves.
 
     The bf16 iteration is chaotic at the last bit: two implementations with the same rounding points that differ
     only in the order of their fp32 accumulations drift apart by about 10x per step (5e-6 after step one, 5e-3
@@ -111,8 +132,108 @@ def test_newton_schulz_full_size_against_oracle(shape):
     want = OO.newton_schulz(u).float()
     to_torch_gpu, to_oracle, torch_gpu_to_oracle = rel_fro(have, torch_gpu), rel_fro(have, want), rel_fro(torch_gpu, want)
     print(f"newton_schulz {shape}: vs torch on this GPU {to_torch_gpu:.3e}, vs CPU oracle {to_oracle:.3e}, torch GPU vs CPU oracle {torch_gpu_to_oracle:.3e}")
+    _report({"test": "newton_schulz", "shape": list(shape), "vs_torch_gpu": to_torch_gpu, "vs_cpu_oracle": to_oracle, "torch_gpu_vs_cpu_oracle": torch_gpu_to_oracle})
     assert to_torch_gpu < MUON_TOL
     assert to_oracle < max(MUON_TOL, 1.1 * torch_gpu_to_oracle)
     # the bulk of the singular values was pushed into the band the quintic iteration converges to
-    s = torch.linalg.svdvals(have[:512].double() @ have[:512].double().T).sqrt()
+    rows = have[:512] if shape[0] <= shape[1] else have[:, :512].T
+    s = torch.linalg.svdvals(rows.double() @ rows.double().T).sqrt()
     assert float(s.max()) < 1.3 and float(s.median()) > 0.5
+
+
+@pytest.mark.parametrize("shape", FULL_SIZE_SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_muon_step_full_size_parameter_delta(shape):
+    """One whole update per shape (fp32 parameter and momentum, bf16-valued gradients): the PARAMETER DELTA against
+    ``torch.optim.Muon.step`` executed on this GPU (the reference's own execution) and against the CPU oracle, the
+    momentum buffer to fp32 rounding."""
+    torch.set_num_threads(16)
+    n = shape[0] * shape[1]
+    p0 = normal_flat(n, 0.02, 41, torch.float32).view(shape)
+    g = normal_flat(n, 1e-3, 42, torch.bfloat16).float().view(shape)
+    buf0 = normal_flat(n, 1e-3, 43, torch.float32).view(shape)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+
+    p_dev, buf_dev = p0.to(DEV), buf0.to(DEV)
+    F.muon_step(p_dev, g.to(DEV), buf_dev, **kw)
+    delta = (p_dev.cpu() - p0)
+
+    p_t = torch.nn.Parameter(p0.to(DEV))
+    opt = torch.optim.Muon([p_t], **kw)
+    opt.state[p_t]["momentum_buffer"] = buf0.to(DEV)
+    p_t.grad = g.to(DEV)
+    opt.step()
+    delta_torch_gpu = p_t.detach().cpu() - p0
+    buf_torch_gpu = opt.state[p_t]["momentum_buffer"].cpu()
+    del opt, p_t
+
+    p_ref, buf_ref = p0.clone(), buf0.clone()
+    OO.muon_step(p_ref, g, buf_ref, **kw)
+    delta_oracle = p_ref - p0
+
+    to_torch_gpu, to_oracle, torch_gpu_to_oracle = rel_fro(delta, delta_torch_gpu), rel_fro(delta, delta_oracle), rel_fro(delta_torch_gpu, delta_oracle)
+    print(f"muon_step {shape}: delta vs torch on this GPU {to_torch_gpu:.3e}, vs CPU oracle {to_oracle:.3e}, torch GPU vs CPU oracle {torch_gpu_to_oracle:.3e}")
+    _report({"test": "muon_step_delta", "shape": list(shape), "vs_torch_gpu": to_torch_gpu, "vs_cpu_oracle": to_oracle, "torch_gpu_vs_cpu_oracle": torch_gpu_to_oracle})
+    assert to_torch_gpu < MUON_TOL
+    assert to_oracle < max(MUON_TOL, 1.1 * torch_gpu_to_oracle)
+    assert torch.allclose(buf_dev.cpu(), buf_ref, rtol=1e-6, atol=1e-9)
+    assert torch.allclose(buf_dev.cpu(), buf_torch_gpu, rtol=1e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("shape", [(512, 768), (768, 512), (1024, 1024)])
+def test_symmetric_tile_variants_forced(shape, variant):
+    """Both tilings of the symmetric products (1: 256 x 256 with mirrored store, 2: 128 x 128) forced on small
+    shapes, where the CPU oracle is cheap; the default chooser is restored afterwards."""
+    from matrix_fsdp_amd import _lib
+
+    u = normal_flat(shape[0] * shape[1], 1e-3, 9, torch.float32).view(shape)
+    want = OO.newton_schulz(u).float()
+    _lib.lib().mfsdp_set_muon_tuning(0, variant, 0, 0, 0, -1)
+    try:
+        have = F.newton_schulz(u.to(DEV)).float().cpu()
+    finally:
+        _lib.lib().mfsdp_set_muon_tuning(0, 3, 0, 0, 0, -1)
+    assert rel_fro(have, want) < MUON_TOL
+
+
+def test_hidden5120_layer_buffer_copies_and_adamw_tail_full_size():
+    """One owner-layout layer buffer of the hidden5120 model at its own size (uneven rank shards, padded staging):
+    pack, unpack and the compact owner gradient fill bit-exact against the oracle; then AdamW on the 41 062 400-element
+    fp32 tail shard of rank 0 at t = 1, 2 against the oracle."""
+    torch.set_num_threads(16)
+    w = HIDDEN5120
+    layer = 1
+    order, specs, plan = reordered_specs(w, layer)
+    assert len(set(plan.shard_sizes)) > 1
+    full = normal_flat(plan.total_numel, 0.02, w.seed + layer, torch.bfloat16)
+    padded = torch.full((w.world_size * plan.max_shard_size,), 3, dtype=torch.bfloat16, device=DEV)
+    pack_program(plan, torch.bfloat16, device=DEV).run((full.to(DEV),), padded)
+    assert_same_bits(padded, CO.pack_to_padded(full, plan))
+    out = torch.full((plan.total_numel,), 5, dtype=torch.bfloat16, device=DEV)
+    unpack_program(plan, torch.bfloat16, device=DEV).run((padded,), out)
+    assert_same_bits(out, full)
+    del padded, out
+
+    by_offset = sorted(specs, key=lambda s: s.offset)
+    grads = [normal_flat(s.numel, 1e-3, w.grad_seed + k, torch.bfloat16) for k, s in enumerate(by_offset)]
+    expect = CO.fill_compact_owner_reduce_scatter_input(
+        by_offset, [g.float() for g in grads], plan.shard_sizes, plan.rank_segments, torch.full((sum(plan.shard_sizes),), -1.0)
+    )
+    offsets = [CO.packed_grad_offset_for_param(s, plan.shard_sizes, plan.rank_segments, compact=True) for s in by_offset]
+    program = compact_owner_program(by_offset, offsets, sum(plan.shard_sizes), torch.bfloat16, torch.float32, device=DEV)
+    packed = torch.full((sum(plan.shard_sizes),), -1.0, device=DEV)
+    program.run([g.to(DEV) for g in grads], packed)
+    assert_same_bits(packed, expect)
+    del packed, expect, grads, full
+
+    n = HIDDEN5120_TAIL_NUMEL
+    assert n == 41_062_400
+    p, m, v = normal_flat(n, 0.02, 7, torch.float32), torch.zeros(n), torch.zeros(n)
+    dev = [t.to(DEV) for t in (p, m, v)]
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for t in (1, 2):
+        g = normal_flat(n, 1e-3, 8 + t, torch.float32)
+        F.adamw_step(dev[0], g.to(DEV), dev[1], dev[2], t, **kw)
+        OO.adamw_step(p, g, m, v, t, **kw)
+        for have, want in zip(dev, (p, m, v)):
+            assert max_err_over_scale(have, want) < 1e-6
