@@ -74,6 +74,28 @@ int mfsdp_copy_rank_segments_to_full(const void* local, int64_t local_numel, voi
                                      const int64_t* numels, int64_t n_segments, int elem_bytes, void* stream);
 
 /*
+ * The same copy with the reference's own metadata contract: the three arrays are DEVICE arrays of n_segments int64
+ * each (the tensors kernels/native.py:470-489 builds once per layout and caches) and max_numel is the longest
+ * segment.  Replaces copy_rank_segments_to_full (matrix_copy.cpp:53-83, matrix_copy_cuda.cu:8-23, 38-67) argument
+ * for argument; enqueue-only: no allocation, no host read of the metadata, no synchronisation, so it may be
+ * captured into a HIP graph.  Offsets o < ceil(max_numel / 256) * 256 of every segment are copied, as the
+ * reference's (tiles, segments) grid does.  The host cannot see the metadata, so the kernel validates it: a segment
+ * with a negative start or size, or one that leaves `local` or `output`, is skipped (the reference would access
+ * out of bounds).  n_segments == 0 or max_numel == 0 returns at once.
+ *
+ * workspace == NULL: one tile slot per (segment, tile index up to max_numel), the reference's launch shape; needs
+ * nothing besides the arguments and is safe on concurrent streams.  workspace != NULL (8-byte aligned, at least
+ * mfsdp_copy_rank_segments_workspace_bytes(n_segments) bytes, not shared by calls that may overlap): a scan kernel
+ * writes the segments' running tile counts there and a persistent grid cuts the copy by bytes instead of by
+ * segment -- the shape to use when segment lengths differ widely.
+ */
+int64_t mfsdp_copy_rank_segments_workspace_bytes(int64_t n_segments);
+int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                                            const int64_t* d_global_starts, const int64_t* d_local_starts,
+                                            const int64_t* d_numels, int64_t n_segments, int64_t max_numel,
+                                            int elem_bytes, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Segment program: a layout's whole copy (every rank, every segment, pad
  * zero-fill, optional dtype conversion) compiled once into device-resident
  * tables and replayed with ONE kernel launch per buffer.

@@ -21,7 +21,7 @@ CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
 DT_F16 = 2  # mfsdp_accumulate only
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class CopyRun(Structure):
@@ -47,6 +47,11 @@ SIGNATURES = {
     "mfsdp_copy_rank_segments_to_full": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int64, c_int, c_void_p],
+    ),
+    "mfsdp_copy_rank_segments_workspace_bytes": (c_int64, [c_int64]),
+    "mfsdp_copy_rank_segments_to_full_device": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p],
     ),
     "mfsdp_merge_segment_runs": (c_int64, [POINTER(CopyRun), c_int64, POINTER(CopyRun)]),
     "mfsdp_segment_program_create": (

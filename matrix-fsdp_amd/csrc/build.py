@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 CSRC = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(CSRC)
 LIB_PATH = os.path.join(PKG, "libmfsdp_hip.so")
-SOURCES = ("common.hip", "segment_copy.hip", "muon_elementwise.hip", "muon_gemm.hip", "muon.hip", "adamw.hip")
+SOURCES = ("common.hip", "segment_copy.hip", "segment_copy_device.hip", "muon_elementwise.hip", "muon_gemm.hip", "muon.hip", "adamw.hip")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",

@@ -1,0 +1,333 @@
+// Rank-segment copy driven by DEVICE-resident metadata: the enqueue-only form of copy_rank_segments_to_full.
+//
+//     output[global_starts[s] + o] = local[local_starts[s] + o]      for o < numels[s], every segment s
+//
+// The three int64 arrays live in device memory (the caller caches them per layout), so the host sees neither the
+// segment sizes nor their alignment: everything a segment needs is derived inside the kernels.
+//
+// Addressing.  For segment s let S and D be the byte addresses of its first source and destination element.  The
+// widest vector both sides can use is V = the largest power of two <= 16 dividing S - D; the copy then runs on the
+// destination's V-byte grid: vector k covers destination bytes [D - lead + kV, D - lead + (k+1)V) with
+// lead = D mod V, so every full vector is V-aligned on both sides, and only the first and the last vector of a segment
+// can be partial (moved byte by byte).  A wavefront moves a tile of 64 * 4 vectors (4 KiB at V = 16) with four
+// independent loads in flight per lane, each wave-level access one contiguous 64 V-byte span.
+//
+// Two launch shapes:
+//   * uniform: one tile slot per (segment, tile index up to the longest segment), as the reference's
+//     (tiles, segments) grid; needs no memory besides the arguments, slots past a segment's end exit at once;
+//   * balanced: a one-workgroup scan writes the running tile count of the segments into a caller-provided scratch
+//     array, and a persistent grid takes chunks of consecutive tiles, finds the chunk's
+//     first segment by bisection and walks on from there -- the work is cut by bytes, so one very long segment
+//     beside many short ones costs no empty slots.
+#include "mfsdp_common.h"
+
+#include <algorithm>
+
+namespace mfsdp {
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kUnroll = 4;
+constexpr int kTileVectors = kWave * kUnroll;
+constexpr int kCopyThreads = 256;
+constexpr int kWavesPerBlock = kCopyThreads / kWave;
+constexpr int kScanThreads = 1024;
+constexpr int kScanPerThread = 8;
+constexpr int kChunkTiles = 8;  // consecutive tiles one bisection serves (32 KiB at V = 16)
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct SegmentCopyArgs {
+  const char* local;
+  char* output;
+  const int64_t* global_starts;
+  const int64_t* local_starts;
+  const int64_t* numels;
+  int64_t local_numel;
+  int64_t output_numel;
+  int64_t n_segments;
+  int64_t limit;  // elements copied per segment at most (the reference's grid covers max_numel rounded up to 256)
+  int elem_bytes;
+};
+
+struct Geometry {
+  const char* src;   // first source byte
+  char* dst;         // first destination byte
+  int64_t nbytes;
+  uint32_t vec;      // V
+  uint32_t lead;     // D mod V
+  uint64_t n_vec;    // vectors on the destination's V-byte grid that hold at least one byte of the segment
+  uint64_t tiles;
+};
+
+// Geometry of segment s; a segment that is empty or leaves either tensor gets zero tiles (it is not copied).
+__device__ __forceinline__ Geometry segment_geometry(const SegmentCopyArgs& a, int64_t s) {
+  Geometry g{};
+  const int64_t gs = a.global_starts[s], ls = a.local_starts[s];
+  int64_t n = a.numels[s];
+  if (n <= 0 || gs < 0 || ls < 0 || ls > a.local_numel - n || gs > a.output_numel - n) return g;
+  n = n < a.limit ? n : a.limit;
+  g.src = a.local + ls * a.elem_bytes;
+  g.dst = a.output + gs * a.elem_bytes;
+  g.nbytes = n * a.elem_bytes;
+  const uint64_t diff = reinterpret_cast<uint64_t>(g.src) - reinterpret_cast<uint64_t>(g.dst);
+  const uint64_t low = diff & (~diff + 1);  // lowest set bit, 0 when the addresses are congruent to every power of two
+  g.vec = (low == 0 || low >= 16) ? 16u : static_cast<uint32_t>(low);
+  g.lead = static_cast<uint32_t>(reinterpret_cast<uint64_t>(g.dst) & (g.vec - 1));
+  g.n_vec = (static_cast<uint64_t>(g.nbytes) + g.lead + g.vec - 1) / g.vec;
+  g.tiles = (g.n_vec + kTileVectors - 1) / kTileVectors;
+  return g;
+}
+
+template <int V>
+struct Vec {
+  uint32_t w[(V + 3) / 4];
+};
+
+template <int V>
+__device__ __forceinline__ Vec<V> load_vec(const char* p) {
+  Vec<V> r;
+  if constexpr (V == 16) {
+    const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
+  } else if constexpr (V == 8) {
+    const u32x2 a = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    r.w[0] = a.x; r.w[1] = a.y;
+  } else if constexpr (V == 4) {
+    r.w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+  } else if constexpr (V == 2) {
+    r.w[0] = *reinterpret_cast<const uint16_t*>(p);
+  } else {
+    r.w[0] = *reinterpret_cast<const uint8_t*>(p);
+  }
+  return r;
+}
+
+template <int V>
+__device__ __forceinline__ void store_vec(char* p, const Vec<V>& v) {
+  if constexpr (V == 16) {
+    const u32x4 a = {v.w[0], v.w[1], v.w[2], v.w[3]};
+    __builtin_nontemporal_store(a, reinterpret_cast<u32x4*>(p));
+  } else if constexpr (V == 8) {
+    const u32x2 a = {v.w[0], v.w[1]};
+    __builtin_nontemporal_store(a, reinterpret_cast<u32x2*>(p));
+  } else if constexpr (V == 4) {
+    __builtin_nontemporal_store(v.w[0], reinterpret_cast<uint32_t*>(p));
+  } else if constexpr (V == 2) {
+    *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(v.w[0]);
+  } else {
+    *reinterpret_cast<uint8_t*>(p) = static_cast<uint8_t>(v.w[0]);
+  }
+}
+
+// Tiles [tile_begin, tile_end) of one segment, by one wavefront.
+template <int V>
+__device__ __forceinline__ void copy_tiles(const Geometry& g, uint64_t tile_begin, uint64_t tile_end, uint32_t lane) {
+  for (uint64_t tile = tile_begin; tile < tile_end; ++tile) {
+    Vec<V> data[kUnroll];
+    int64_t at[kUnroll];  // byte offset of the vector from the segment's first byte; < 0 or cut at the end: partial
+    bool full[kUnroll], partial[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint64_t k = tile * kTileVectors + static_cast<uint64_t>(u) * kWave + lane;
+      at[u] = static_cast<int64_t>(k) * V - static_cast<int64_t>(g.lead);
+      const bool live = k < g.n_vec;
+      full[u] = live && at[u] >= 0 && at[u] + V <= g.nbytes;
+      partial[u] = live && !full[u];
+      if (full[u]) data[u] = load_vec<V>(g.src + at[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (full[u]) store_vec<V>(g.dst + at[u], data[u]);
+      if (partial[u]) {  // the first or the last vector of the segment
+        const int64_t b0 = at[u] < 0 ? 0 : at[u];
+        const int64_t b1 = at[u] + V < g.nbytes ? at[u] + V : g.nbytes;
+        for (int64_t b = b0; b < b1; ++b) g.dst[b] = g.src[b];
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void copy_tiles_any(const Geometry& g, uint64_t tile_begin, uint64_t tile_end, uint32_t lane) {
+  switch (g.vec) {
+    case 16: copy_tiles<16>(g, tile_begin, tile_end, lane); break;
+    case 8: copy_tiles<8>(g, tile_begin, tile_end, lane); break;
+    case 4: copy_tiles<4>(g, tile_begin, tile_end, lane); break;
+    case 2: copy_tiles<2>(g, tile_begin, tile_end, lane); break;
+    default: copy_tiles<1>(g, tile_begin, tile_end, lane); break;
+  }
+}
+
+// ---- uniform launch shape: slot = (segment, j) with j < slots_per_segment, the tile count of the longest segment at
+// V = 16; the slot's wave moves tiles j, j + slots_per_segment, ... of its segment (more than one only when the
+// segment's addresses force a narrower vector).
+__global__ void __launch_bounds__(kCopyThreads)
+segment_copy_uniform_kernel(SegmentCopyArgs a, uint64_t slots_per_segment, uint64_t n_slots) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWavesPerBlock;
+  const uint32_t wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps the metadata loads scalar
+  for (uint64_t slot = static_cast<uint64_t>(blockIdx.x) * kWavesPerBlock + wave_in_block; slot < n_slots; slot += n_waves) {
+    const uint64_t s = slot / slots_per_segment;
+    const uint64_t first = slot - s * slots_per_segment;
+    const Geometry g = segment_geometry(a, static_cast<int64_t>(s));
+    for (uint64_t tile = first; tile < g.tiles; tile += slots_per_segment) copy_tiles_any(g, tile, tile + 1, lane);
+  }
+}
+
+// ---- balanced launch shape, step 1: prefix[0] = 0, prefix[s + 1] = tiles of segments 0..s.  One workgroup.
+__global__ void __launch_bounds__(kScanThreads)
+segment_tile_scan_kernel(SegmentCopyArgs a, uint64_t* __restrict__ prefix) {
+  __shared__ uint64_t wave_sums[kScanThreads / kWave];
+  __shared__ uint64_t block_total;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  uint64_t carry = 0;
+  if (tid == 0) prefix[0] = 0;
+  for (int64_t base = 0; base < a.n_segments; base += static_cast<int64_t>(kScanThreads) * kScanPerThread) {
+    const int64_t first = base + static_cast<int64_t>(tid) * kScanPerThread;
+    uint64_t mine[kScanPerThread];
+    uint64_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+      mine[i] = first + i < a.n_segments ? segment_geometry(a, first + i).tiles : 0;
+      sum += mine[i];
+    }
+    // inclusive scan of the per-thread sums: within the wave by shuffles, across the 16 waves through LDS
+    uint64_t incl = sum;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const uint64_t up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sums[wave] = incl;
+    __syncthreads();
+    uint64_t before = carry;
+    for (int w = 0; w < wave; ++w) before += wave_sums[w];
+    if (tid == kScanThreads - 1) block_total = before + incl - carry;
+    uint64_t running = before + incl - sum;  // tiles of every segment before this thread's first
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+      running += mine[i];
+      if (first + i < a.n_segments) prefix[first + i + 1] = running;
+    }
+    __syncthreads();
+    carry += block_total;
+    __syncthreads();  // wave_sums / block_total are rewritten by the next round
+  }
+}
+
+// ---- balanced launch shape, step 2: persistent waves take chunks of consecutive tiles.
+__global__ void __launch_bounds__(kCopyThreads)
+segment_copy_balanced_kernel(SegmentCopyArgs a, const uint64_t* __restrict__ prefix, uint32_t chunk_tiles) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * kWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWavesPerBlock;
+  const uint64_t total = prefix[a.n_segments];
+  const uint64_t n_chunks = (total + chunk_tiles - 1) / chunk_tiles;
+  for (uint64_t chunk = wave; chunk < n_chunks; chunk += n_waves) {
+    uint64_t t = chunk * chunk_tiles;
+    const uint64_t t_end = t + chunk_tiles < total ? t + chunk_tiles : total;
+    // the segment holding tile t: prefix[s] <= t < prefix[s + 1]  (prefix[0] = 0 <= t < total = prefix[n_segments])
+    int64_t lo = 0, hi = a.n_segments;
+    while (hi - lo > 1) {
+      const int64_t mid = lo + ((hi - lo) >> 1);
+      if (prefix[mid] <= t) lo = mid; else hi = mid;
+    }
+    int64_t s = lo;
+    while (t < t_end && s < a.n_segments) {
+      const uint64_t seg_begin = prefix[s], seg_end = prefix[s + 1];
+      if (t >= seg_end) { ++s; continue; }
+      const Geometry g = segment_geometry(a, s);
+      const uint64_t upto = t_end < seg_end ? t_end : seg_end;
+      copy_tiles_any(g, t - seg_begin, upto - seg_begin, lane);
+      t = upto;
+    }
+  }
+}
+
+int check_args(const void* local, int64_t local_numel, void* output, int64_t output_numel, const int64_t* d_global_starts,
+               const int64_t* d_local_starts, const int64_t* d_numels, int64_t n_segments, int64_t max_numel, int elem_bytes) {
+  if (n_segments < 0) return fail(MFSDP_ERR_INVALID, "n_segments must be non-negative");
+  if (max_numel < 0) return fail(MFSDP_ERR_INVALID, "max_numel must be non-negative");
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return fail(MFSDP_ERR_INVALID, "elem_bytes must be 1, 2, 4 or 8, got %d", elem_bytes);
+  if (local_numel < 0 || output_numel < 0) return fail(MFSDP_ERR_INVALID, "tensor sizes must be non-negative");
+  if (n_segments > 0 && max_numel > 0) {
+    if (!d_global_starts || !d_local_starts || !d_numels) return fail(MFSDP_ERR_INVALID, "segment metadata is null");
+    if (!local || !output) return fail(MFSDP_ERR_INVALID, "local or output is null");
+    if ((reinterpret_cast<uintptr_t>(local) | reinterpret_cast<uintptr_t>(output)) % elem_bytes)
+      return fail(MFSDP_ERR_INVALID, "local and output must be aligned to the element size");
+  }
+  return MFSDP_OK;
+}
+
+SegmentCopyArgs make_args(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                          const int64_t* d_global_starts, const int64_t* d_local_starts, const int64_t* d_numels,
+                          int64_t n_segments, int64_t max_numel, int elem_bytes) {
+  SegmentCopyArgs a{};
+  a.local = static_cast<const char*>(local);
+  a.output = static_cast<char*>(output);
+  a.global_starts = d_global_starts;
+  a.local_starts = d_local_starts;
+  a.numels = d_numels;
+  a.local_numel = local_numel;
+  a.output_numel = output_numel;
+  a.n_segments = n_segments;
+  // the reference launches ceil(max_numel / 256) blocks of 256 threads per segment (matrix_copy_cuda.cu:45-51):
+  // offsets below that many elements are copied, whatever numels[s] says
+  a.limit = (max_numel + 255) / 256 * 256;
+  a.elem_bytes = elem_bytes;
+  return a;
+}
+
+// Upper bound of the tiles one segment can need: V >= elem_bytes, plus one vector for a misaligned start.
+uint64_t max_tiles_per_segment(const SegmentCopyArgs& a) {
+  const uint64_t vectors = static_cast<uint64_t>(a.limit) + 1;
+  return (vectors + kTileVectors - 1) / kTileVectors;
+}
+
+int launch_balanced(const SegmentCopyArgs& a, uint64_t* prefix, hipStream_t stream) {
+  hipLaunchKernelGGL(segment_tile_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, a, prefix);
+  MFSDP_CHECK_LAUNCH("segment_tile_scan_kernel");
+  const uint64_t bound = static_cast<uint64_t>(a.n_segments) * max_tiles_per_segment(a);
+  const uint64_t want = (bound + kChunkTiles * kWavesPerBlock - 1) / (kChunkTiles * kWavesPerBlock);
+  const uint64_t cap = static_cast<uint64_t>(device_cu_count()) * 4;
+  const dim3 grid(static_cast<uint32_t>(std::max<uint64_t>(1, std::min(want, cap))));
+  hipLaunchKernelGGL(segment_copy_balanced_kernel, grid, dim3(kCopyThreads), 0, stream, a, prefix, static_cast<uint32_t>(kChunkTiles));
+  MFSDP_CHECK_LAUNCH("segment_copy_balanced_kernel");
+  return MFSDP_OK;
+}
+
+}  // namespace
+}  // namespace mfsdp
+
+using namespace mfsdp;
+
+extern "C" int64_t mfsdp_copy_rank_segments_workspace_bytes(int64_t n_segments) {
+  return n_segments < 0 ? 0 : (n_segments + 1) * 8;
+}
+
+extern "C" int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                                                       const int64_t* d_global_starts, const int64_t* d_local_starts,
+                                                       const int64_t* d_numels, int64_t n_segments, int64_t max_numel,
+                                                       int elem_bytes, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = check_args(local, local_numel, output, output_numel, d_global_starts, d_local_starts, d_numels, n_segments, max_numel, elem_bytes)) return rc;
+  if (n_segments == 0 || max_numel == 0) return MFSDP_OK;
+  const SegmentCopyArgs a = make_args(local, local_numel, output, output_numel, d_global_starts, d_local_starts, d_numels, n_segments, max_numel, elem_bytes);
+  if (workspace != nullptr) {
+    if (workspace_bytes < mfsdp_copy_rank_segments_workspace_bytes(n_segments))
+      return fail(MFSDP_ERR_INVALID, "workspace of %lld bytes needed for %lld segments, got %lld",
+                  static_cast<long long>(mfsdp_copy_rank_segments_workspace_bytes(n_segments)), static_cast<long long>(n_segments),
+                  static_cast<long long>(workspace_bytes));
+    if (reinterpret_cast<uintptr_t>(workspace) % 8) return fail(MFSDP_ERR_INVALID, "workspace must be 8-byte aligned");
+    return launch_balanced(a, static_cast<uint64_t*>(workspace), as_stream(stream));
+  }
+  // tiles of the longest segment when its addresses allow 16-byte vectors (one more vector for a misaligned start)
+  const uint64_t per_segment = (static_cast<uint64_t>(a.limit) * elem_bytes / 16 + kTileVectors) / kTileVectors;
+  const uint64_t n_slots = static_cast<uint64_t>(n_segments) * per_segment;
+  const uint64_t want = (n_slots + kWavesPerBlock - 1) / kWavesPerBlock;
+  const dim3 grid(static_cast<uint32_t>(std::min<uint64_t>(want, (uint64_t{1} << 31) - 1)));
+  hipLaunchKernelGGL(segment_copy_uniform_kernel, grid, dim3(kCopyThreads), 0, as_stream(stream), a, per_segment, n_slots);
+  MFSDP_CHECK_LAUNCH("segment_copy_uniform_kernel");
+  return MFSDP_OK;
+}

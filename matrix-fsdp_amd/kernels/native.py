@@ -100,6 +100,79 @@ def native_copy_rank_segments_to_full(
     return True
 
 
+# (device type, device index, segment triples) -> (global_starts, local_starts, numels, max_numel), created once per
+# layout and kept for the life of the process, as the reference keeps them (kernels/native.py:20-23, 470-489)
+_SEGMENT_METADATA_CACHE: dict[tuple, tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]] = {}
+
+
+def _segment_metadata_tensors(segments: tuple[LayoutSegment, ...], *, device: torch.device):
+    key = (device.type, device.index, tuple((s.global_start, s.local_start, s.numel) for s in segments))
+    cached = _SEGMENT_METADATA_CACHE.get(key)
+    if cached is None:
+        columns = [[s.global_start for s in segments], [s.local_start for s in segments], [s.numel for s in segments]]
+        tensors = [torch.tensor(c, dtype=torch.int64, device=device) for c in columns]
+        cached = (*tensors, max(columns[2], default=0))
+        _SEGMENT_METADATA_CACHE[key] = cached
+    return cached
+
+
+def copy_rank_segments_to_full(
+    local_tensor: torch.Tensor,
+    output_tensor: torch.Tensor,
+    global_starts: torch.Tensor,
+    local_starts: torch.Tensor,
+    numels: torch.Tensor,
+    max_numel: int,
+    *,
+    workspace: torch.Tensor | None = None,
+) -> None:
+    """The extension function of the reference, argument for argument
+    (kernels/native/matrix_copy.cpp:53-83): device int64 metadata tensors, enqueue
+    only on the current stream, the reference's checks as ``RuntimeError``.
+    ``workspace`` (uint8, ``mfsdp_copy_rank_segments_workspace_bytes`` long)
+    selects the byte-balanced launch shape."""
+    for t, name in ((local_tensor, "local_tensor"), (output_tensor, "output_tensor"), (global_starts, "global_starts"),
+                    (local_starts, "local_starts"), (numels, "numels")):
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a CUDA tensor")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    for t, name in ((global_starts, "global_starts"), (local_starts, "local_starts"), (numels, "numels")):
+        if t.dtype != torch.int64:
+            raise RuntimeError(f"{name} must be int64")
+    if local_tensor.dim() != 1:
+        raise RuntimeError("local_tensor must be 1D")
+    if output_tensor.dim() != 1:
+        raise RuntimeError("output_tensor must be 1D")
+    if local_tensor.dtype != output_tensor.dtype:
+        raise RuntimeError("source and destination dtype mismatch")
+    if global_starts.numel() != local_starts.numel() or global_starts.numel() != numels.numel():
+        raise RuntimeError("metadata length mismatch")
+    if max_numel < 0:
+        raise RuntimeError("max_numel must be non-negative")
+    if global_starts.numel() == 0:
+        return
+    ws_ptr, ws_bytes = (None, 0)
+    if workspace is not None:
+        if not workspace.is_cuda or not workspace.is_contiguous() or workspace.device != output_tensor.device:
+            raise RuntimeError("workspace must be a contiguous CUDA tensor on the output's device")
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    stream = torch.cuda.current_stream(output_tensor.device).cuda_stream
+    with torch.cuda.device(output_tensor.device):
+        _lib.check(
+            _lib.lib().mfsdp_copy_rank_segments_to_full_device(
+                local_tensor.data_ptr(), local_tensor.numel(), output_tensor.data_ptr(), output_tensor.numel(),
+                global_starts.data_ptr(), local_starts.data_ptr(), numels.data_ptr(), global_starts.numel(), int(max_numel),
+                local_tensor.element_size(), ws_ptr, ws_bytes, stream,
+            )
+        )
+
+
+def copy_rank_segments_workspace(n_segments: int, device) -> torch.Tensor:
+    """Scratch for the byte-balanced launch shape of ``copy_rank_segments_to_full``."""
+    return torch.empty(int(_lib.lib().mfsdp_copy_rank_segments_workspace_bytes(n_segments)), dtype=torch.uint8, device=device)
+
+
 def native_copy_rank_chunk_from_packed(
     packed_rank_chunks: torch.Tensor,
     output_tensor: torch.Tensor,

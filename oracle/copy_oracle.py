@@ -15,6 +15,10 @@ Pinning (what makes this oracle trustworthy, see tests/test_oracle_*.py):
   * the 2x2 block layout is checked against the strided-slice closed form;
   * casts are checked against ``Tensor.to`` over crafted bit patterns;
   * round trips and write-exactly-once invariants on random layouts;
+  * ``copy_rank_segments_to_full_kernel`` is checked against a literal thread
+    by thread walk of the reference kernel's grid on small inputs, and against
+    ``copy_local_rank_segments`` (pinned by the reference vectors) whenever
+    ``max_numel`` covers every segment;
   * the checkpoint redistribution (``target_local_shard_from_full`` etc.) is
     checked against the pinned pack / unpack functions: a rank's shard of the
     full buffer is that rank's slice of the packed order, on random layouts.
@@ -127,6 +131,21 @@ def copy_local_rank_segments(local: torch.Tensor, output: torch.Tensor, segments
     matrix_fsdp/kernels/native/matrix_copy_cuda.cu:8-23)."""
     for seg in segments:
         output[seg.global_start : seg.global_end].copy_(local[seg.local_start : seg.local_start + _numel(seg)])
+
+
+def copy_rank_segments_to_full_kernel(local: torch.Tensor, output: torch.Tensor, global_starts, local_starts, numels, max_numel: int) -> None:
+    """The extension function as its kernel executes it
+    (matrix_fsdp/kernels/native/matrix_copy_cuda.cu:8-23, 38-51): a grid of
+    ``ceil(max_numel / 256)`` blocks of 256 threads per segment, thread
+    ``offset`` copying one element when ``offset < numel``.  With
+    ``max_numel >= max(numels)`` (what the caller passes,
+    kernels/native.py:484) this is ``copy_local_rank_segments``; a smaller
+    ``max_numel`` leaves the tail of longer segments uncopied."""
+    covered = (int(max_numel) + 255) // 256 * 256
+    for g, l, n in zip(global_starts, local_starts, numels):
+        n = min(int(n), covered)
+        if n > 0:
+            output[int(g) : int(g) + n].copy_(local[int(l) : int(l) + n])
 
 
 # ---------------------------------------------------------------- P7

@@ -127,6 +127,41 @@ def test_two_rank_gather_and_reduce_semantics(golden):
         assert torch.equal(out / 2, f32(expect))
 
 
+def test_kernel_form_of_the_rank_segment_copy_against_a_literal_grid_walk():
+    """``copy_rank_segments_to_full_kernel``: every (block, thread) of the reference's launch
+    (matrix_copy_cuda.cu:8-23, 45-51) visited one by one on small inputs."""
+    gen = torch.Generator().manual_seed(5)
+    for trial in range(12):
+        n_seg = int(torch.randint(1, 6, (1,), generator=gen))
+        numels = [int(torch.randint(0, 700, (1,), generator=gen)) for _ in range(n_seg)]
+        local_starts, cursor = [], 0
+        for n in numels:
+            local_starts.append(cursor)
+            cursor += n
+        order = torch.randperm(n_seg, generator=gen).tolist()
+        global_starts, gcursor = [0] * n_seg, 3
+        for i in order:
+            global_starts[i] = gcursor
+            gcursor += numels[i] + 2
+        local = torch.arange(cursor, dtype=torch.float32) + 1
+        max_numel = max(numels) if trial % 3 else max(numels) // 2  # every third trial: a max_numel that is too small
+        want = torch.zeros(gcursor)
+        threads, tiles = 256, (max_numel + 255) // 256
+        for segment in range(n_seg):  # blockIdx.y
+            for block in range(tiles):  # blockIdx.x
+                for thread in range(threads):
+                    offset = block * threads + thread
+                    if offset < numels[segment]:
+                        want[global_starts[segment] + offset] = local[local_starts[segment] + offset]
+        have = torch.zeros(gcursor)
+        O.copy_rank_segments_to_full_kernel(local, have, global_starts, local_starts, numels, max_numel)
+        assert torch.equal(have, want)
+        if max_numel >= max(numels):
+            via_slices = torch.zeros(gcursor)
+            O.copy_local_rank_segments(local, via_slices, segs([[(g, g + n, l) for g, l, n in zip(global_starts, local_starts, numels)]])[0])
+            assert torch.equal(have, via_slices)
+
+
 def test_padded_gather_and_unpad():
     sizes = (4, 6, 0, 3)
     shards = [torch.arange(n, dtype=torch.float32) + 10 * r for r, n in enumerate(sizes)]
