@@ -96,6 +96,21 @@ int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_num
                                             int elem_bytes, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * The device-metadata copy above in its byte-balanced launch shape, for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
+ * segments' running tile counts go into a 1 MiB array that is part of the library's device image (every GPU the
+ * library runs on holds its own copy until the process ends) instead of a caller's workspace, so the call neither
+ * allocates nor frees anything; more than MFSDP_NOALLOC_MAX_SEGMENTS segments are rejected with
+ * MFSDP_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two
+ * streams) race and must use mfsdp_copy_rank_segments_to_full_device with their own workspaces instead.
+ */
+#define MFSDP_NOALLOC_MAX_SEGMENTS 131071
+int mfsdp_copy_rank_segments_to_full_noalloc(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                                             const int64_t* d_global_starts, const int64_t* d_local_starts,
+                                             const int64_t* d_numels, int64_t n_segments, int64_t max_numel,
+                                             int elem_bytes, void* stream);
+
+/*
  * Segment program: a layout's whole copy (every rank, every segment, pad
  * zero-fill, optional dtype conversion) compiled once into device-resident
  * tables and replayed with ONE kernel launch per buffer.

@@ -22,6 +22,7 @@ DT_F32 = 0
 DT_BF16 = 1
 DT_F16 = 2  # mfsdp_accumulate only
 ABI_VERSION = 2
+NOALLOC_MAX_SEGMENTS = 131071  # MFSDP_NOALLOC_MAX_SEGMENTS
 
 
 class CopyRun(Structure):
@@ -52,6 +53,10 @@ SIGNATURES = {
     "mfsdp_copy_rank_segments_to_full_device": (
         c_int,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p],
+    ),
+    "mfsdp_copy_rank_segments_to_full_noalloc": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p],
     ),
     "mfsdp_merge_segment_runs": (c_int64, [POINTER(CopyRun), c_int64, POINTER(CopyRun)]),
     "mfsdp_segment_program_create": (

@@ -15,13 +15,14 @@
 // Two launch shapes:
 //   * uniform: one tile slot per (segment, tile index up to the longest segment), as the reference's
 //     (tiles, segments) grid; needs no memory besides the arguments, slots past a segment's end exit at once;
-//   * balanced: a one-workgroup scan writes the running tile count of the segments into a caller-provided scratch
-//     array, and a persistent grid takes chunks of consecutive tiles, finds the chunk's
+//   * balanced: a one-workgroup scan writes the running tile count of the segments into a caller-provided (or the
+//     library's static) scratch array, and a persistent grid takes chunks of consecutive tiles, finds the chunk's
 //     first segment by bisection and walks on from there -- the work is cut by bytes, so one very long segment
 //     beside many short ones costs no empty slots.
 #include "mfsdp_common.h"
 
 #include <algorithm>
+#include <mutex>
 
 namespace mfsdp {
 namespace {
@@ -34,6 +35,13 @@ constexpr int kWavesPerBlock = kCopyThreads / kWave;
 constexpr int kScanThreads = 1024;
 constexpr int kScanPerThread = 8;
 constexpr int kChunkTiles = 8;  // consecutive tiles one bisection serves (32 KiB at V = 16)
+constexpr int kMaxDevices = 64;
+
+// Scratch of the entry point that allocates nothing: the running tile counts of up to kStaticMaxSegments segments.
+constexpr int64_t kStaticScratchBytes = 1 << 20;
+constexpr int64_t kStaticMaxSegments = kStaticScratchBytes / 8 - 1;
+static_assert(kStaticMaxSegments == MFSDP_NOALLOC_MAX_SEGMENTS, "the header states the limit");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -298,6 +306,24 @@ int launch_balanced(const SegmentCopyArgs& a, uint64_t* prefix, hipStream_t stre
   return MFSDP_OK;
 }
 
+// Device address of the static scratch array, looked up once per device (each device holds its own copy).
+int static_scratch(uint64_t** out) {
+  static std::mutex mu;
+  static uint64_t* cached[kMaxDevices] = {nullptr};
+  int dev = 0;
+  MFSDP_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MFSDP_ERR_UNSUPPORTED, "device index %d is beyond the %d devices the static scratch covers", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (cached[dev] == nullptr) {
+    void* ptr = nullptr;
+    MFSDP_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(MFSDP_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch");
+    cached[dev] = static_cast<uint64_t*>(ptr);
+  }
+  *out = cached[dev];
+  return MFSDP_OK;
+}
+
 }  // namespace
 }  // namespace mfsdp
 
@@ -330,4 +356,19 @@ extern "C" int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_
   hipLaunchKernelGGL(segment_copy_uniform_kernel, grid, dim3(kCopyThreads), 0, as_stream(stream), a, per_segment, n_slots);
   MFSDP_CHECK_LAUNCH("segment_copy_uniform_kernel");
   return MFSDP_OK;
+}
+
+extern "C" int mfsdp_copy_rank_segments_to_full_noalloc(const void* local, int64_t local_numel, void* output, int64_t output_numel,
+                                                        const int64_t* d_global_starts, const int64_t* d_local_starts,
+                                                        const int64_t* d_numels, int64_t n_segments, int64_t max_numel,
+                                                        int elem_bytes, void* stream) {
+  if (int rc = check_args(local, local_numel, output, output_numel, d_global_starts, d_local_starts, d_numels, n_segments, max_numel, elem_bytes)) return rc;
+  if (n_segments > kStaticMaxSegments)
+    return fail(MFSDP_ERR_UNSUPPORTED, "the static scratch holds the tile counts of at most %lld segments, got %lld",
+                static_cast<long long>(kStaticMaxSegments), static_cast<long long>(n_segments));
+  if (n_segments == 0 || max_numel == 0) return MFSDP_OK;
+  uint64_t* prefix = nullptr;
+  if (int rc = static_scratch(&prefix)) return rc;
+  const SegmentCopyArgs a = make_args(local, local_numel, output, output_numel, d_global_starts, d_local_starts, d_numels, n_segments, max_numel, elem_bytes);
+  return launch_balanced(a, prefix, as_stream(stream));
 }
