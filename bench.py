@@ -34,6 +34,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 NS_COEFFS = (3.4445, -4.7750, 2.0315)
+# figures taken from the committed rocprofv3 counter profiles (they cannot be measured from inside this process)
+PROFILED_TRAFFIC = {"bytes_per_launch": 812_800_000, "source": "profiles/segment_program_hbm_traffic.md"}
 
 
 def parse_args():
@@ -44,7 +46,8 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=0, help="layer buffers of the hidden4096 workload (0 = all 32)")
     ap.add_argument("--skip-legs", action="store_true", help="only the timed pack/unpack region (used under rocprofv3)")
     ap.add_argument("--skip-mixed", action="store_true", help="skip the hidden5120 mixed-step leg")
-    ap.add_argument("--legs", default="rows,muon,adamw,mixed", help="comma list of the extra legs to run: rows (hidden2048 row split), muon, adamw, mixed")
+    ap.add_argument("--legs", default="ceiling,rows,muon,adamw,mixed",
+                    help="comma list of the extra legs to run: ceiling (plain copy / read-only / write-only probes), rows (hidden2048 row split), muon, adamw, mixed")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
     ap.add_argument("--no-launch-events", action="store_true", help="no HIP events inside the timed region (launch time from the wall clock)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -100,7 +103,8 @@ def main() -> int:
     _lib.lib()  # fail loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    host_threads = min(os.cpu_count() or 1, 16)
+    host_cores = os.cpu_count() or 1
+    host_threads = min(host_cores, 16)  # torch's CPU kernels stop scaling beyond that on these copies
     torch.set_num_threads(host_threads)
 
     # ------------------------------------------------------------------ timed region: hidden4096 2x2 block pack + unpack
@@ -166,9 +170,10 @@ def main() -> int:
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for a
-        # plain 1 GiB copy in the same run (measured once, profiles/segment_program_hbm_traffic.md)
-        "traffic": 812_800_000 if layers > 0 else None,
+        # HBM bytes per launch: not measurable from inside the run; the figure of the committed counter profile of this
+        # workload (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain 1 GiB copy), quoted only for the run it describes
+        "traffic": PROFILED_TRAFFIC["bytes_per_launch"] if layers == w.layers else None,
+        "traffic_source": PROFILED_TRAFFIC["source"] if layers == w.layers else None,
         "algorithmic_bytes_per_launch": bytes_per_launch,
         "avg_launch_ms": round(avg_launch_ms, 5),
         "launches_timed": len(launch_events) * 2 * layers,
@@ -204,6 +209,41 @@ def main() -> int:
         want.discard("mixed")
     if "mixed" in want:
         want |= {"muon", "adamw"}  # the mixed step reuses their set-up
+    if "ceiling" in want:
+        # -------------------------------------------------------------- what this part sustains: a plain contiguous copy of one
+        # layer buffer's size through the library's range copy, pure reads and pure writes in the same launch shape
+        import ctypes
+
+        n_el = w.total_numel
+        a_buf = torch.empty(n_el, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02)
+        b_buf = torch.empty(n_el, dtype=torch.bfloat16, device=dev)
+        sink = torch.zeros(4096, dtype=torch.uint8, device=dev)
+        from matrix_fsdp_amd.kernels import native as N
+
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        nbytes = 2 * n_el
+
+        def probe(kind):
+            _lib.check(_lib.lib().mfsdp_hbm_probe(kind, a_buf.data_ptr(), (sink if kind == 0 else b_buf).data_ptr(), nbytes, stream))
+
+        t_copy, _ = time_launches(torch, lambda: N.copy_range(a_buf, b_buf, 0), 20, 5)
+        t_read, _ = time_launches(torch, lambda: probe(0), 20, 5)
+        t_write, _ = time_launches(torch, lambda: probe(1), 20, 5)
+        t_torch, _ = time_launches(torch, lambda: b_buf.copy_(a_buf), 20, 5)
+        read_gbps, write_gbps = nbytes / (t_read * 1e-3) / 1e9, nbytes / (t_write * 1e-3) / 1e9
+        legs["hbm_ceiling_one_layer_buffer"] = {
+            "plain_copy_GBps": round(2 * nbytes / (t_copy * 1e-3) / 1e9, 1),
+            "read_only_GBps": round(read_gbps, 1),
+            "write_only_GBps": round(write_gbps, 1),
+            "equal_mix_of_both_GBps": round(2 / (1 / read_gbps + 1 / write_gbps), 1),
+            "torch_copy_GBps": round(2 * nbytes / (t_torch * 1e-3) / 1e9, 1),
+            "note": f"{nbytes} bytes each way, contiguous; plain copy = mfsdp_copy_range (read + written bytes counted), probes = "
+            "mfsdp_hbm_probe; the equal mix is the rate at which half the bytes move at the read-only and half at the write-only rate",
+        }
+        result["roofline"]["frac_of_plain_copy"] = round(achieved / legs["hbm_ceiling_one_layer_buffer"]["plain_copy_GBps"], 4)
+        del a_buf, b_buf, sink
+        torch.cuda.empty_cache()
+
     if "rows" in want:
         # -------------------------------------------------------------- hidden2048 row split: pack / unpack / chunk-cat + cast
         w2 = HIDDEN2048_W4
@@ -228,6 +268,10 @@ def main() -> int:
             ("pack", all_layers(lambda i: pack2.run((full2[i],), gath2[i])), pack2.bytes_moved),
             ("unpack", all_layers(lambda i: unpack2.run((gath2[i],), out2[i])), unpack2.bytes_moved),
             ("chunk_cat_bf16_to_f32", all_layers(lambda i: fill2.run(grads2[i], packed32[i])), fill2.bytes_moved),
+            # the same eight buffers as ONE grid (mfsdp_segment_program_run_many): launch ramp and tail paid once
+            ("pack_8_buffers_one_grid", lambda: pack2.run_many([(f,) for f in full2], gath2), pack2.bytes_moved),
+            ("unpack_8_buffers_one_grid", lambda: unpack2.run_many([(g,) for g in gath2], out2), unpack2.bytes_moved),
+            ("chunk_cat_bf16_to_f32_8_buffers_one_grid", lambda: fill2.run_many(grads2, packed32), fill2.bytes_moved),
         ):
             med, _ = time_launches(torch, fn, 20, 5)
             legs[f"hidden2048_w4_rows.{name}"] = {
@@ -373,7 +417,8 @@ def main() -> int:
         result["cpu_baseline"] = {
             "value": round(cpu_gbps, 3),
             "unit": "GB/s",
-            "cores": host_threads,
+            "cores": host_cores,
+            "threads": host_threads,
             "kind": "port",
             "sample": f"{reps} x (pack + unpack) of ONE of the 32 hidden4096 layer buffers ({w.total_numel} bf16 elements, ~85k row segments) with the "
             "oracle's per-segment slice-copy loops; same byte accounting as the GPU value",
@@ -391,7 +436,8 @@ def main() -> int:
             result["cpu_baseline_muon"] = {
                 "value": round(fl / t_ns / 1e12, 4),
                 "unit": "TFLOP/s",
-                "cores": host_threads,
+                "cores": host_cores,
+                "threads": host_threads,
                 "kind": "port",
                 "sample": f"{ns_reps} x 5-step Newton-Schulz of one 4096x4096 matrix with the oracle (torch bf16 matmuls on the CPU)",
                 "seconds": round(t_ns, 2),

@@ -14,7 +14,8 @@
  *     mfsdp_last_error() holds a message for the calling thread.  A binding
  *     turns non-zero into the host language's exception (the reference's
  *     TORCH_CHECK -> RuntimeError convention, matrix_copy.cpp:60-78, 86-94);
- *   - only the *_create / *_destroy calls allocate or free device memory.
+ *   - only the *_create / *_destroy calls and the host-metadata mfsdp_copy_rank_segments_to_full allocate or
+ *     free device memory.
  *
  * Element offsets, not bytes, everywhere; `elem_bytes` in {1, 2, 4, 8}.
  */
@@ -153,11 +154,13 @@ typedef struct mfsdp_segment_program mfsdp_segment_program;
 int64_t mfsdp_merge_segment_runs(const mfsdp_copy_run* segs, int64_t n_segs, mfsdp_copy_run* out);
 
 /*
- * Validates the runs against the extents (src_numels[n_srcs], dst_numel),
- * compiles and uploads them.  Allocates device memory; synchronous.
- * `convert` is one of MFSDP_CONVERT_*; elem_bytes is the element size for
- * MFSDP_CONVERT_NONE (ignored otherwise: 2 -> 4 or 4 -> 2 bytes: bf16 or fp16 on
- * the 2-byte side).
+ * Validates the runs against the extents (src_numels[n_srcs], dst_numel), refuses runs whose destination rows
+ * overlap (the reference's sequential slice writes make an overlap well defined; the waves of one launch write in
+ * no particular order), compiles the tables for every vector width a later run may need and uploads them.
+ * Allocates device memory; synchronous.  `convert` is one of MFSDP_CONVERT_*; elem_bytes is the element size for
+ * MFSDP_CONVERT_NONE (ignored otherwise: 2 -> 4 or 4 -> 2 bytes: bf16 or fp16 on the 2-byte side).  Any number of
+ * sources: fill_reduce_scatter_input (runtime/grad_bucket.py:71-116) takes any number of gradients; a launch
+ * carries 128 source pointers, so a program over more sources replays as one launch per block of 128.
  */
 int mfsdp_segment_program_create(const mfsdp_copy_run* runs, int64_t n_runs,
                                  const int64_t* src_numels, int32_t n_srcs, int64_t dst_numel,
@@ -170,17 +173,38 @@ int64_t mfsdp_segment_program_num_runs(const mfsdp_segment_program* program);
 /*
  * Replays the program: srcs[i] is the device base of source i and must hold
  * at least the src_numels[i] elements given at create time, dst at least
- * dst_numel.  One kernel launch, no allocation, no synchronisation (the first
- * call with base pointers less aligned than any earlier call compiles a
- * narrower-vector variant of the tables; that one call allocates).
+ * dst_numel.  One kernel launch per vector width in use (one for a layout whose
+ * offsets are all 16-byte multiples); never allocates, never synchronises.  Base
+ * pointers less aligned than the layout run the same tables at a narrower
+ * vector width.
  */
 int mfsdp_segment_program_run(mfsdp_segment_program* program, const void* const* srcs, int32_t n_srcs,
                               void* dst, void* stream);
 
-/* Launch tuning for experiments: blocks per CU of the persistent copy grid
- * (0 = library default), non-temporal hints (0 none, 1 loads and stores, 2 loads only, 3 stores only, -1 = default) and
- * 128-bit loads in flight per lane (4 or 8; applies to programs created afterwards). */
-void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll);
+/*
+ * The same program over n_buffers buffers of one layout in ONE grid (the layer buffers of a step that are
+ * due together: prefetched all-gather outputs, the gradient buckets of a backward window): buffer b reads
+ * srcs[b * n_srcs + i] and writes dsts[b].  The per-launch ramp and tail are paid once instead of n_buffers times.
+ * Both pointer tables travel in the kernel arguments (128 source pointers, 64 destinations): larger batches are
+ * split into several launches.  Never allocates, never synchronises.
+ */
+int mfsdp_segment_program_run_many(mfsdp_segment_program* program, int32_t n_buffers, const void* const* srcs,
+                                   int32_t n_srcs, void* const* dsts, void* stream);
+
+/* Launch tuning for experiments (safe to call while other threads launch): workgroups per CU of the copy grid
+ * (-1 = library default, 0 = one workgroup per four tiles without a grid-stride loop, n > 0 = persistent grid of n
+ * per CU), non-temporal hints (0 none, 1 loads and stores, 2 loads only, 3 stores only, -1 = default); and, for
+ * programs created afterwards, 128-bit loads in flight per lane (1, 2 or 4; 0 = default); threads per workgroup (64, 128
+ * or 256: the 256 lanes of a tile spread over 4, 2 or 1 workgroups; 0 = default). */
+void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll, int block_threads);
+
+/*
+ * Measurement aid (no counterpart in the reference): one pass of pure reads (kind 0: `bytes` of src are loaded
+ * and discarded; dst is a 4 KiB sink that is never written as long as src holds no all-ones 16-byte group) or pure
+ * writes (kind 1: `bytes` of dst are filled with a constant), one workgroup per 4 KiB like the copy kernels, so that a
+ * benchmark can state what the part sustains in each direction beside the copy it measures.
+ */
+int mfsdp_hbm_probe(int kind, const void* src, void* dst, int64_t bytes, void* stream);
 
 /* ------------------------------------------------------------------ cast */
 

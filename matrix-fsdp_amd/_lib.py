@@ -21,7 +21,7 @@ CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
 DT_F16 = 2  # mfsdp_accumulate only
-ABI_VERSION = 2
+ABI_VERSION = 3
 NOALLOC_MAX_SEGMENTS = 131071  # MFSDP_NOALLOC_MAX_SEGMENTS
 
 
@@ -67,7 +67,9 @@ SIGNATURES = {
     "mfsdp_segment_program_bytes": (c_int64, [c_void_p]),
     "mfsdp_segment_program_num_runs": (c_int64, [c_void_p]),
     "mfsdp_segment_program_run": (c_int, [c_void_p, POINTER(c_void_p), c_int32, c_void_p, c_void_p]),
-    "mfsdp_set_copy_tuning": (None, [c_int, c_int, c_int]),
+    "mfsdp_segment_program_run_many": (c_int, [c_void_p, c_int32, POINTER(c_void_p), c_int32, POINTER(c_void_p), c_void_p]),
+    "mfsdp_set_copy_tuning": (None, [c_int, c_int, c_int, c_int]),
+    "mfsdp_hbm_probe": (c_int, [c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "mfsdp_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mfsdp_muon_workspace_bytes": (c_int64, [c_int64, c_int64]),
     "mfsdp_newton_schulz": (

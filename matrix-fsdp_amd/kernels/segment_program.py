@@ -42,8 +42,6 @@ RUN_DTYPE = np.dtype(
 )
 assert RUN_DTYPE.itemsize == ctypes.sizeof(_lib.CopyRun)
 
-MAX_SOURCES = 128
-
 _CONVERT_CODES = {
     (torch.bfloat16, torch.float32): _lib.CONVERT_BF16_TO_F32,
     (torch.float32, torch.bfloat16): _lib.CONVERT_F32_TO_BF16,
@@ -98,7 +96,8 @@ def merge_runs(runs: np.ndarray) -> np.ndarray:
 
 class SegmentProgram:
     """Owns one ``mfsdp_segment_program``.  ``run`` is one kernel launch on
-    the current HIP stream; it neither allocates nor synchronises."""
+    the current HIP stream (one per block of 128 sources and per vector width
+    in use); it neither allocates nor synchronises."""
 
     def __init__(
         self,
@@ -118,8 +117,6 @@ class SegmentProgram:
             convert, elem_bytes = _CONVERT_CODES[(src_dtype, dst_dtype)], 0
         else:
             raise RuntimeError(f"segment programs convert bfloat16 / float16 <-> float32 only, got {src_dtype} -> {dst_dtype}.")
-        if len(src_numels) > MAX_SOURCES:
-            raise RuntimeError(f"a segment program reads at most {MAX_SOURCES} sources, got {len(src_numels)}.")
         self.src_dtype, self.dst_dtype = src_dtype, dst_dtype
         self.src_numels = tuple(int(n) for n in src_numels)
         self.dst_numel = int(dst_numel)
@@ -164,6 +161,36 @@ class SegmentProgram:
                 _lib.lib().mfsdp_segment_program_run(self._handle, self._src_array, len(self.src_numels), dst.data_ptr(), stream)
             )
         return dst
+
+    def run_many(self, srcs_per_buffer: Sequence[Sequence[torch.Tensor]], dsts: Sequence[torch.Tensor]) -> None:
+        """The program over several buffers of this layout in one grid
+        (``mfsdp_segment_program_run_many``): buffer ``b`` reads
+        ``srcs_per_buffer[b]`` and writes ``dsts[b]``."""
+        if self._handle is None:
+            raise RuntimeError("segment program was destroyed.")
+        if len(srcs_per_buffer) != len(dsts):
+            raise RuntimeError(f"{len(srcs_per_buffer)} source lists for {len(dsts)} destinations.")
+        if not dsts:
+            return
+        n_srcs = len(self.src_numels)
+        src_array = (ctypes.c_void_p * max(1, n_srcs * len(dsts)))()
+        dst_array = (ctypes.c_void_p * len(dsts))()
+        device = dsts[0].device
+        for b, (srcs, dst) in enumerate(zip(srcs_per_buffer, dsts)):
+            if len(srcs) != n_srcs:
+                raise RuntimeError(f"segment program expects {n_srcs} sources, got {len(srcs)} (buffer {b}).")
+            _check_tensor(dst, self.dst_dtype, self.dst_numel, f"destination {b}")
+            if dst.device != device:
+                raise RuntimeError("every buffer of a batch must be on one device.")
+            dst_array[b] = dst.data_ptr()
+            for i, (t, n) in enumerate(zip(srcs, self.src_numels)):
+                _check_tensor(t, self.src_dtype, n, f"source {i} of buffer {b}")
+                if t.device != device:
+                    raise RuntimeError("sources and destination must be on one device.")
+                src_array[b * n_srcs + i] = t.data_ptr()
+        stream = torch.cuda.current_stream(device).cuda_stream
+        with torch.cuda.device(device):
+            _lib.check(_lib.lib().mfsdp_segment_program_run_many(self._handle, len(dsts), src_array, n_srcs, dst_array, stream))
 
     def destroy(self) -> None:
         if getattr(self, "_handle", None) is not None:

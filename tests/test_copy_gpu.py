@@ -287,6 +287,98 @@ def test_random_grad_copy_in_with_cast():
         assert_same_bits(packed, expect)
 
 
+def test_grad_copy_in_with_three_hundred_gradients():
+    """fill_reduce_scatter_input takes any number of gradients (runtime/grad_bucket.py:71-116): a root unit that
+    keeps what no layer manages easily holds more parameters than one launch carries pointers for."""
+    rng = random.Random(3)
+    world = 4
+    sizes = [rng.choice([1, 7, 64, 300, 1024, 4099]) for _ in range(300)]
+    params = params_from_pairs([(f"p{i}", n) for i, n in enumerate(sizes)])
+    total = sum(sizes)
+    for plan in (contiguous_even_plan(total, world), random_plan(rng, total, world)):
+        grads_cpu = [torch.randn(n, generator=torch.Generator().manual_seed(i)).bfloat16() for i, n in enumerate(sizes)]
+        expect = torch.full((world * plan.max_shard_size,), 3.0)
+        O.fill_reduce_scatter_input(params, grads_cpu, plan.shard_sizes, plan.rank_segments, total, expect)
+        program = grad_fill_program(params, plan.shard_sizes, plan.rank_segments, torch.bfloat16, torch.float32, device=DEV)
+        packed = torch.full((world * plan.max_shard_size,), 5.0, device=DEV)
+        program.run([g.to(DEV) for g in grads_cpu], packed)
+        assert_same_bits(packed, expect)
+
+
+def test_run_many_matches_run_buffer_by_buffer():
+    """One grid over several buffers of a layout: pack, unpack and the gradient copy-in, with more buffers than one
+    launch carries destinations for (64) and more source pointers than it carries (128)."""
+    rng = random.Random(4)
+    total, world = 5000, 3
+    plan = random_plan(rng, total, world)
+    pack = pack_program(plan, torch.bfloat16, device=DEV)
+    unpack = unpack_program(plan, torch.bfloat16, device=DEV)
+    n_buffers = 70
+    fulls = [(torch.randperm(total, generator=torch.Generator().manual_seed(b)) % 251 + 1).to(torch.bfloat16) for b in range(n_buffers)]
+    dev_fulls = [f.to(DEV) for f in fulls]
+    padded = [torch.full((world * plan.max_shard_size,), 7, dtype=torch.bfloat16, device=DEV) for _ in range(n_buffers)]
+    pack.run_many([(f,) for f in dev_fulls], padded)
+    outs = [torch.full((total,), 9, dtype=torch.bfloat16, device=DEV) for _ in range(n_buffers)]
+    unpack.run_many([(p,) for p in padded], outs)
+    for b in range(n_buffers):
+        assert_same_bits(padded[b], O.pack_to_padded(fulls[b], plan))
+        assert_same_bits(outs[b], fulls[b])
+    sizes = [rng.randint(1, 400) for _ in range(9)]
+    params = params_from_pairs([(f"p{i}", n) for i, n in enumerate(sizes)])
+    gplan = random_plan(rng, sum(sizes), world)
+    fill = grad_fill_program(params, gplan.shard_sizes, gplan.rank_segments, torch.bfloat16, torch.float32, device=DEV)
+    n_buffers = 20  # 180 source pointers: two launches
+    grads = [[torch.randn(n, generator=torch.Generator().manual_seed(100 * b + i)).bfloat16() for i, n in enumerate(sizes)] for b in range(n_buffers)]
+    packed = [torch.full((world * gplan.max_shard_size,), 5.0, device=DEV) for _ in range(n_buffers)]
+    fill.run_many([[g.to(DEV) for g in gs] for gs in grads], packed)
+    for b in range(n_buffers):
+        expect = torch.full((world * gplan.max_shard_size,), 3.0)
+        O.fill_reduce_scatter_input(params, grads[b], gplan.shard_sizes, gplan.rank_segments, sum(sizes), expect)
+        assert_same_bits(packed[b], expect)
+    with pytest.raises(RuntimeError, match="source lists"):
+        pack.run_many([(dev_fulls[0],)], padded[:2])
+
+
+def test_base_pointers_less_aligned_than_the_layout_run_the_same_tables():
+    """A program compiled for 16-byte groups replayed on views that start 2, 4, 6, ... bytes into their allocations
+    (narrower vector width, same tables: no table is built at run time), for plain copies and for the widening and
+    narrowing conversions."""
+    w = MLP_W2
+    plan = w.plan()
+    full = normal_flat(w.total_numel, 0.02, 5, torch.bfloat16)
+    want_padded = O.pack_to_padded(full, plan)
+    pack = pack_program(plan, torch.bfloat16, device=DEV)
+    unpack = unpack_program(plan, torch.bfloat16, device=DEV)
+    n_padded = w.world_size * plan.max_shard_size
+    for src_shift, dst_shift in ((0, 0), (1, 0), (0, 1), (2, 4), (3, 5), (4, 4), (7, 1)):
+        src = torch.zeros(w.total_numel + src_shift, dtype=torch.bfloat16, device=DEV)[src_shift:]
+        src.copy_(full)
+        guard = torch.full((n_padded + dst_shift + 8,), 3, dtype=torch.bfloat16, device=DEV)
+        dst = guard[dst_shift : dst_shift + n_padded]
+        free_before = torch.cuda.mem_get_info()[0]
+        pack.run((src,), dst)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert_same_bits(dst, want_padded)
+        assert bool((guard[:dst_shift] == 3).all()) and bool((guard[dst_shift + n_padded :] == 3).all())
+        back = torch.zeros(w.total_numel + src_shift, dtype=torch.bfloat16, device=DEV)[src_shift:]
+        unpack.run((dst,), back)
+        assert_same_bits(back, full)
+    fill = grad_fill_program(w.specs, plan.shard_sizes, plan.rank_segments, torch.bfloat16, torch.float32, device=DEV)
+    grads_cpu = [normal_flat(s.numel, 1e-3, 6 + i, torch.bfloat16) for i, s in enumerate(w.specs)]
+    expect = torch.full((n_padded,), 3.0)
+    O.fill_reduce_scatter_input(w.specs, grads_cpu, plan.shard_sizes, plan.rank_segments, w.total_numel, expect)
+    for shift in (0, 1, 2, 3):
+        grads = []
+        for g in grads_cpu:
+            holder = torch.zeros(g.numel() + shift, dtype=torch.bfloat16, device=DEV)[shift:]
+            holder.copy_(g)
+            grads.append(holder)
+        packed = torch.full((n_padded + shift,), 5.0, device=DEV)[shift:]
+        fill.run(grads, packed)
+        assert_same_bits(packed, expect)
+
+
 @pytest.mark.parametrize("world", [2, 3, 4])
 def test_chunk_cat_with_ragged_params(world):
     sizes = [5, 6, 1, 16, 33, world, 3 * world + 1, 4096 + 3]

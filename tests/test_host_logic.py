@@ -198,6 +198,63 @@ def test_merge_runs_builds_strided_blocks():
     assert merge_runs(make_runs([], [], [])).shape[0] == 0
 
 
+def test_program_create_rejects_overlapping_destination_rows():
+    """The validation of ``mfsdp_segment_program_create`` runs on the host before anything touches a device: two
+    interleaved column blocks of one matrix are legal (their bounding spans overlap, no row does), every true overlap
+    is refused with MFSDP_ERR_INVALID.  Without a device a legal program fails later, at the upload (MFSDP_ERR_HIP)."""
+    from matrix_fsdp_amd.kernels import segment_program as SP
+
+    handle = _lib.lib()
+
+    def create(rows):
+        runs = np.zeros(len(rows), dtype=SP.RUN_DTYPE)
+        for i, (src_off, dst_off, row_len, n_rows, src_stride, dst_stride) in enumerate(rows):
+            runs[i] = (src_off, dst_off, row_len, n_rows, src_stride, dst_stride, 0, 0)
+        numels = (ctypes.c_int64 * 1)(1 << 20)
+        out = ctypes.c_void_p()
+        rc = handle.mfsdp_segment_program_create(
+            runs.ctypes.data_as(ctypes.POINTER(_lib.CopyRun)), len(rows), numels, 1, 1 << 20, _lib.CONVERT_NONE, 2, ctypes.byref(out)
+        )
+        if rc == 0:
+            handle.mfsdp_segment_program_destroy(out)
+        return rc, handle.mfsdp_last_error().decode()
+
+    legal = (0, 2)  # built (a device is present) or refused by the upload only
+    # left and right half of a 64 x 32 matrix as two strided runs
+    assert create([(0, 0, 16, 64, 16, 32), (4096, 16, 16, 64, 16, 32)])[0] in legal
+    # three runs that interleave row by row, given in any order
+    assert create([(0, 20, 10, 50, 10, 30), (1000, 0, 10, 50, 10, 30), (2000, 10, 10, 50, 10, 30)])[0] in legal
+    # a plain segment that starts exactly where the last row of a strided run ends
+    assert create([(0, 0, 16, 64, 16, 32), (4096, 32 * 63 + 16, 17, 1, 0, 0)])[0] in legal
+    # a plain segment between two rows of a strided run
+    assert create([(0, 0, 16, 64, 16, 32), (4096, 16 + 32 * 7, 16, 1, 0, 0)])[0] in legal
+    for rows in (
+        [(0, 0, 16, 64, 16, 32), (4096, 15, 16, 64, 16, 32)],          # shifted by one element: every row overlaps
+        [(0, 0, 100, 1, 0, 0), (500, 99, 5, 1, 0, 0)],                 # plain segments, one element shared
+        [(0, 0, 16, 64, 16, 32), (4096, 32 * 40 + 8, 4, 1, 0, 0)],     # a short segment inside row 40
+        [(0, 0, 10, 3, 10, 100), (500, 205, 10, 1, 0, 0)],             # only the last row is hit
+    ):
+        rc, message = create(rows)
+        assert rc == 1 and "two runs write destination offset" in message, (rows, rc, message)
+    # against brute force on random small programs
+    rng = np.random.default_rng(0)
+    seen = {True: 0, False: 0}
+    for _ in range(400):
+        rows, hits, clash = [], np.zeros(4096, dtype=np.int32), False
+        for _ in range(int(rng.integers(2, 6))):
+            row_len, n_rows = int(rng.integers(1, 12)), int(rng.integers(1, 9))
+            stride = row_len + int(rng.integers(0, 20)) if n_rows > 1 else 0
+            dst_off = int(rng.integers(0, 300))
+            rows.append((0, dst_off, row_len, n_rows, row_len, stride))
+            for r in range(n_rows):
+                hits[dst_off + r * stride : dst_off + r * stride + row_len] += 1
+        clash = bool((hits > 1).any())
+        seen[clash] += 1
+        rc, _ = create(rows)
+        assert (rc == 1) == clash, (rows, rc)
+    assert min(seen.values()) > 50
+
+
 def test_fill_runs_cover_exactly_the_gaps():
     fills = fill_runs_for_gaps(make_runs([0, 0], [2, 8], [3, 2]), 12)
     assert [(int(f["dst_off"]), int(f["row_len"]), int(f["src_id"])) for f in fills] == [(0, 2, -1), (5, 3, -1), (10, 2, -1)]
