@@ -36,6 +36,13 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 NS_COEFFS = (3.4445, -4.7750, 2.0315)
 # figures taken from the committed rocprofv3 counter profiles (they cannot be measured from inside this process)
 PROFILED_TRAFFIC = {"bytes_per_launch": 812_800_000, "source": "profiles/segment_program_hbm_traffic.md"}
+PROFILED_MUON = {
+    # SQ_VALU_MFMA_BUSY_CYCLES over the SIMD cycles of the dispatch, per tile shape
+    "mfma_busy": {"gemm_nt_kernel<256,256> (general products)": 0.524, "gemm_nt_kernel<128,128> (symmetric products)": 0.446},
+    # the dominant launch, B X on 12288 x 4096 (768 workgroups): FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, in bytes
+    "traffic_bytes_per_launch": (2 * 344_237 + 176_947) * 1024,
+    "source": "profiles/gemm_nt_kernel_muon_hidden4096_counters.md, profiles/gemm_nt_kernel_muon_hbm_traffic.md",
+}
 
 
 def parse_args():
@@ -320,14 +327,26 @@ def main() -> int:
         }
         result["muon_ns_TFLOPs"] = round(tflops, 1)
         result["muon_ms_per_step"] = round(med, 4)
+        executed = sum(int(_lib.lib().mfsdp_muon_executed_flops(sh[0], sh[1], 5)) for sh in MUON_HIDDEN4096_SHAPES)
+        tflops_executed = executed / (med * 1e-3) / 1e12
+        legs["muon_hidden4096"]["ns_TFLOPs_executed"] = round(tflops_executed, 1)
         result["roofline_muon"] = {
-            "kernel": "gemm_nt_kernel (Newton-Schulz products, whole Muon step timed)",
+            "kernel": "gemm_nt_kernel (Newton-Schulz products; the whole Muon step is timed: momentum, norm, 15 products per matrix, update)",
             "bound": "mfma",
+            # the reference's count: full GEMMs, 5 * (4 m^2 n + 2 m^3) per matrix
             "achieved": round(tflops, 1),
             "peak": BF16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "frac_reference_count": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4),
+            # flops the kernels execute: the symmetric products X X^T and A A compute the tiles on or below the diagonal only
+            "achieved_executed": round(tflops_executed, 1),
+            "frac_executed": round(tflops_executed / BF16_MFMA_PEAK_TFLOPS, 4),
+            "executed_over_reference_flops": round(executed / flops, 4),
+            # counter figures of the committed profiles of this leg (they cannot be measured from inside this process)
+            "mfma_busy": PROFILED_MUON["mfma_busy"],
+            "traffic": PROFILED_MUON["traffic_bytes_per_launch"],
+            "traffic_source": PROFILED_MUON["source"],
         }
         del mats
         torch.cuda.empty_cache()

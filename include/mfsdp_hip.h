@@ -232,6 +232,13 @@ int mfsdp_accumulate(void* dst, const void* src, int64_t numel, int dtype, void*
 int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols);
 
 /*
+ * Flops the Newton-Schulz kernels execute for `steps` iterations on a rows x cols matrix with the current tuning
+ * (operands zero-padded to multiples of 256; the two symmetric products of a step compute only the tiles on or below
+ * the diagonal).  The reference executes full products: steps * (4 m^2 n + 2 m^3) with m the short side.
+ */
+int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps);
+
+/*
  * Quintic Newton-Schulz orthogonalisation of one matrix, the arithmetic of
  * torch.optim._muon._zeropower_via_newtonschulz (torch/optim/_muon.py:31-70)
  * that MixedMuonAdamWOptimizer.step reaches through torch.optim.Muon

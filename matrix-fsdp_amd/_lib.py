@@ -72,6 +72,7 @@ SIGNATURES = {
     "mfsdp_hbm_probe": (c_int, [c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "mfsdp_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mfsdp_muon_workspace_bytes": (c_int64, [c_int64, c_int64]),
+    "mfsdp_muon_executed_flops": (c_int64, [c_int64, c_int64, c_int]),
     "mfsdp_newton_schulz": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_float, c_float, c_float, c_int, c_float, c_void_p, c_void_p, c_int64, c_void_p],

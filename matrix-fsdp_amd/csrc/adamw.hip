@@ -75,7 +75,7 @@ adamw_kernel(float* __restrict__ param, const void* __restrict__ grad, float* __
     f32x4 p[U], m[U], v[U], g[U], vmax[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t i = base + u * 256;
+      const int64_t i = base + u * blockDim.x;
       if (i < n_vec) {
         p[u] = ld<NT>(reinterpret_cast<const f32x4*>(param) + i);
         m[u] = ld<NT>(reinterpret_cast<const f32x4*>(exp_avg) + i);
@@ -94,7 +94,7 @@ adamw_kernel(float* __restrict__ param, const void* __restrict__ grad, float* __
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t i = base + u * 256;
+      const int64_t i = base + u * blockDim.x;
       if (i < n_vec) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -156,19 +156,21 @@ extern "C" int mfsdp_adamw_step_ex(float* param, const void* grad, int grad_dtyp
   a.eps = static_cast<float>(eps);
   a.grad_sign = maximize ? -1.0f : 1.0f;
   const int64_t n_vec = vec_ok ? numel / 4 : 0;
-  // four vectors per thread with non-temporal accesses (every byte is touched once), and one workgroup per 16 KiB
-  // block of each stream rather than a persistent grid: workgroups are dispatched in order, so the ones running at
-  // any moment sweep neighbouring addresses of all seven streams.  41 M elements: 5.92 TB/s, against 5.71 TB/s for
-  // 16 persistent workgroups per CU striding over the tensor, 5.0 TB/s for one vector per thread and 5.1-5.5 TB/s
-  // with cached loads or stores; eight vectors per thread spill.
-  constexpr int kVectorsPerThread = 4;
-  const int64_t work = std::max<int64_t>((n_vec + kVectorsPerThread - 1) / kVectorsPerThread, numel - n_vec * 4);
-  const int64_t want = std::max<int64_t>(1, (work + 255) / 256);
+  // Non-temporal accesses (every byte is touched once) and one small workgroup per block of each stream rather than a
+  // persistent grid: workgroups are dispatched in order, so the ones running at any moment sweep neighbouring
+  // addresses of all seven streams, and the finer the workgroups the more evenly loads and stores mix.  41 M
+  // elements: one wavefront per workgroup with two vectors per thread 6.22 TB/s (one vector 5.55, four 6.01; 256 threads
+  // with four vectors 5.93, with two 5.94; 16 persistent workgroups per CU 5.71); 5.1-5.5 TB/s with cached loads or
+  // stores.
+  constexpr int threads = 64, per_thread = 2;
+  const int64_t work = std::max<int64_t>((n_vec + per_thread - 1) / per_thread, numel - n_vec * 4);
+  const int64_t want = std::max<int64_t>(1, (work + threads - 1) / threads);
   const int64_t cap = (int64_t{1} << 31) - 1;  // the loops stride by the grid, so a capped grid stays correct
   const dim3 grid(static_cast<uint32_t>(std::min(want, cap)));
-#define MFSDP_ADAMW(BF16_, AMS_)                                                                                  \
-  hipLaunchKernelGGL((adamw_kernel<BF16_, kVectorsPerThread, true, AMS_>), grid, dim3(256), 0, as_stream(stream), \
+#define MFSDP_ADAMW_U(BF16_, AMS_, U_)                                                                                  \
+  hipLaunchKernelGGL((adamw_kernel<BF16_, U_, true, AMS_>), grid, dim3(threads), 0, as_stream(stream), \
                      param, grad, exp_avg, exp_avg_sq, max_exp_avg_sq, n_vec, numel, a)
+#define MFSDP_ADAMW(BF16_, AMS_) MFSDP_ADAMW_U(BF16_, AMS_, per_thread)
   const bool bf16 = grad_dtype == MFSDP_BF16;
   if (max_exp_avg_sq != nullptr) {
     if (bf16) MFSDP_ADAMW(true, true); else MFSDP_ADAMW(false, true);
@@ -176,6 +178,7 @@ extern "C" int mfsdp_adamw_step_ex(float* param, const void* grad, int grad_dtyp
     if (bf16) MFSDP_ADAMW(true, false); else MFSDP_ADAMW(false, false);
   }
 #undef MFSDP_ADAMW
+#undef MFSDP_ADAMW_U
   MFSDP_CHECK_LAUNCH("adamw_kernel");
   return MFSDP_OK;
 }

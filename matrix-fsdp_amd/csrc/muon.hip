@@ -126,6 +126,16 @@ extern "C" int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols) {
   return plan_workspace(rows, cols, nullptr, &w) ? w.bytes : 0;
 }
 
+extern "C" int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps) {
+  Workspace w;
+  if (steps < 0 || !plan_workspace(rows, cols, nullptr, &w)) return 0;
+  GemmNtArgs gram{}, poly{}, update{};
+  gram.M = gram.N = w.mp; gram.K = w.np; gram.symmetric = 1;
+  poly.M = poly.N = poly.K = w.mp; poly.symmetric = 1;
+  update.M = w.mp; update.N = w.np; update.K = w.mp;
+  return steps * (gemm_nt_executed_flops(gram) + gemm_nt_executed_flops(poly) + gemm_nt_executed_flops(update));
+}
+
 extern "C" int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t rows, int64_t cols, float a, float b, float c,
                                    int steps, float eps, void* out_bf16, void* workspace, int64_t workspace_bytes, void* stream) {
   Workspace w;

@@ -44,6 +44,10 @@ struct GemmTuning {
 void set_gemm_tuning(const GemmTuning& tuning);
 GemmTuning get_gemm_tuning();
 
+// Flops the kernels execute for this product with the current tuning: 2 * tile area * K per computed tile (a symmetric
+// product computes the tiles on or below the diagonal only).
+int64_t gemm_nt_executed_flops(const GemmNtArgs& args);
+
 // Enqueues the GEMM on `stream`; returns an MFSDP_* status.
 int gemm_nt_bf16(const GemmNtArgs& args, const GemmScratch& scratch, hipStream_t stream);
 

@@ -21,6 +21,7 @@
 #include "mfsdp_common.h"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace mfsdp {
@@ -392,78 +393,109 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   }
 }
 
-// Sums the K pieces of every split tile in split order and applies the epilogue of gemm_nt_kernel.
+// Sums the K pieces of every split tile in split order and applies the epilogue of gemm_nt_kernel.  A workgroup
+// finishes a 64 x 64 block of a tile: thread t owns four consecutive columns of rows t / 16, t / 16 + 16, ...; the
+// transposed / mirrored copy goes through LDS so that both orientations leave in whole 16-byte, row-contiguous stores.
 template <int BM, int BN>
 __global__ void __launch_bounds__(256)
 splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
-  constexpr int kGroupsPerTile = BM * BN / 4;  // float4 groups along a row
-  const int tile = blockIdx.x / (kGroupsPerTile / 256);
-  const int group = (blockIdx.x % (kGroupsPerTile / 256)) * 256 + threadIdx.x;
-  const int lrow = group / (BN / 4);
-  const int lcol = (group % (BN / 4)) * 4;
+  constexpr int kSub = 64;
+  constexpr int kSubsPerTile = (BM / kSub) * (BN / kSub);
+  __shared__ __attribute__((aligned(16))) uint16_t transposed[kSub][kSub + 8];
+  const int tile = blockIdx.x / kSubsPerTile;
+  const int sub = blockIdx.x % kSubsPerTile;
+  const int sub_row0 = (sub / (BN / kSub)) * kSub, sub_col0 = (sub % (BN / kSub)) * kSub;
   int tm, tn;
   tile_coords<4>(sched.full_tiles + tile, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
-  const int row = tm * BM + lrow;
-  const int col = tn * BN + lcol;
-  const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
-  // four loads in flight at a time; the sum itself stays in split order
-  f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-  int s = 0;
-  for (; s + 4 <= sched.splits; s += 4) {
-    f32x4 v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s + u) * (BM * BN));
-#pragma unroll
-    for (int u = 0; u < 4; ++u) sum += v[u];
-  }
-  for (; s < sched.splits; ++s) sum += *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN));
   const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
   uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
   int ldct = a.ldct;
-  if (a.symmetric) {
+  if (a.symmetric) {  // mirror the off-diagonal tile
     CT = tm != tn ? C : nullptr;
     ldct = a.ldc;
   }
-  float v[4] = {a.alpha * sum.x, a.alpha * sum.y, a.alpha * sum.z, a.alpha * sum.w};
-  if (D != nullptr) {
-    const u32x2 d = *reinterpret_cast<const u32x2*>(D + static_cast<int64_t>(row) * a.ldd + col);
-    v[0] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x));
-    v[1] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x >> 16));
-    v[2] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y));
-    v[3] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y >> 16));
+  const int t = threadIdx.x;
+  const int lcol = sub_col0 + (t % 16) * 4;
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    const int lrow = sub_row0 + rr * 16 + t / 16;
+    const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
+    // four loads in flight at a time; the sum itself stays in split order
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    int s = 0;
+    for (; s + 4 <= sched.splits; s += 4) {
+      f32x4 piece[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) piece[u] = *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s + u) * (BM * BN));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) sum += piece[u];
+    }
+    for (; s < sched.splits; ++s) sum += *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN));
+    const int row = tm * BM + lrow, col = tn * BN + lcol;
+    float v[4] = {a.alpha * sum.x, a.alpha * sum.y, a.alpha * sum.z, a.alpha * sum.w};
+    if (D != nullptr) {
+      const u32x2 d = *reinterpret_cast<const u32x2*>(D + static_cast<int64_t>(row) * a.ldd + col);
+      v[0] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x));
+      v[1] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x >> 16));
+      v[2] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y));
+      v[3] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y >> 16));
+    }
+    const uint32_t lo = pack_bf16x2(v[0], v[1]);
+    const uint32_t hi = pack_bf16x2(v[2], v[3]);
+    if (!a.skip_c) {
+      const u32x2 packed = {lo, hi};
+      *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
+    }
+    if (CT != nullptr) {
+      const int c = (t % 16) * 4, r = rr * 16 + t / 16;
+      transposed[c][r] = static_cast<uint16_t>(lo);
+      transposed[c + 1][r] = static_cast<uint16_t>(lo >> 16);
+      transposed[c + 2][r] = static_cast<uint16_t>(hi);
+      transposed[c + 3][r] = static_cast<uint16_t>(hi >> 16);
+    }
   }
-  const uint32_t lo = pack_bf16x2(v[0], v[1]);
-  const uint32_t hi = pack_bf16x2(v[2], v[3]);
-  u32x2 packed = {lo, hi};
-  if (!a.skip_c) *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
-  if (CT != nullptr) {
-    CT[static_cast<int64_t>(col) * ldct + row] = static_cast<uint16_t>(lo);
-    CT[static_cast<int64_t>(col + 1) * ldct + row] = static_cast<uint16_t>(lo >> 16);
-    CT[static_cast<int64_t>(col + 2) * ldct + row] = static_cast<uint16_t>(hi);
-    CT[static_cast<int64_t>(col + 3) * ldct + row] = static_cast<uint16_t>(hi >> 16);
+  if (CT == nullptr) return;
+  __syncthreads();
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int r = half * 32 + t / 8, chunk = t % 8;  // row of the transposed block = column of the tile
+    *reinterpret_cast<u32x4*>(CT + static_cast<int64_t>(tn * BN + sub_col0 + r) * ldct + tm * BM + sub_row0 + chunk * 8) =
+        *reinterpret_cast<const u32x4*>(&transposed[r][chunk * 8]);
   }
 }
 
 GemmTuning g_tuning;
+std::mutex g_tuning_mutex;  // the setter may be called while other threads launch: every launch works on one snapshot
+
+GemmTuning tuning_snapshot() {
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  return g_tuning;
+}
+
+// Tiles a product computes: every tile of a general product, the tiles on or below the diagonal of a symmetric one.
+int tile_count(const GemmNtArgs& a, int bm, int bn) {
+  const int tm = a.M / bm, tn = a.N / bn;
+  return a.symmetric ? tm * (tm + 1) / 2 : tm * tn;
+}
 
 template <int BM, int BN, int WM, int WN, int BK, int STAGES, int OCC>
-int launch(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
+int launch(const GemmNtArgs& a, const GemmScratch& scratch, const GemmTuning& tuning, hipStream_t stream) {
   constexpr int blocks_per_cu = OCC;
   Schedule s{};
   s.tiles_m = a.M / BM;
   s.tiles_n = a.N / BN;
-  const int tiles = a.symmetric ? s.tiles_m * (s.tiles_m + 1) / 2 : s.tiles_m * s.tiles_n;
+  const int tiles = tile_count(a, BM, BN);
   const int slots = device_cu_count() * blocks_per_cu;
   const int k_slabs = a.K / BK;
   s.full_tiles = tiles;
   s.splits = 1;
   s.partials = static_cast<float*>(scratch.partials);
-  s.stagger = g_tuning.stagger;
+  s.stagger = tuning.stagger;
   const int rem = tiles % slots;
-  if (g_tuning.split_remainder && rem != 0 && scratch.partials != nullptr) {
+  if (tuning.split_remainder && rem != 0 && scratch.partials != nullptr) {
     // fill the machine once more with pieces of the leftover tiles; cap the pieces per tile so that the summing stays short
-    int splits = std::min({slots / rem, k_slabs, g_tuning.max_splits});
+    int splits = std::min({slots / rem, k_slabs, tuning.max_splits});
     const int64_t tile_bytes = static_cast<int64_t>(BM) * BN * 4;
     while (splits > 1 && static_cast<int64_t>(rem) * splits * tile_bytes > scratch.partials_bytes) --splits;
     if (splits > 1) {
@@ -477,41 +509,32 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) 
   constexpr size_t smem_epilogue = smem_c > smem_ct ? smem_c : smem_ct;
   constexpr size_t smem = smem_loop > smem_epilogue ? smem_loop : smem_epilogue;
   auto kernel = gemm_nt_kernel<BM, BN, WM, WN, BK, STAGES, OCC>;
-  static bool configured = false;  // raising the dynamic LDS limit is needed once per kernel
-  if (!configured) {
-    MFSDP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(smem)));
-    configured = true;
+  {
+    // raising the dynamic LDS limit is needed once per kernel and device
+    static std::mutex mu;
+    static bool configured[64] = {false};
+    int dev = 0;
+    MFSDP_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev < 0 || dev >= 64 || !configured[dev]) {
+      MFSDP_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(smem)));
+      if (dev >= 0 && dev < 64) configured[dev] = true;
+    }
   }
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WM * WN * 64), smem, stream, a, s);
   MFSDP_CHECK_LAUNCH("gemm_nt_kernel");
   if (s.splits > 1) {
-    const int fix_blocks = (tiles - s.full_tiles) * (BM * BN / 4 / 256);
+    const int fix_blocks = (tiles - s.full_tiles) * (BM / 64) * (BN / 64);
     hipLaunchKernelGGL((splitk_fixup_kernel<BM, BN>), dim3(fix_blocks), dim3(256), 0, stream, a, s);
     MFSDP_CHECK_LAUNCH("splitk_fixup_kernel");
   }
   return MFSDP_OK;
 }
 
-}  // namespace
-
-void set_gemm_tuning(const GemmTuning& t) { g_tuning = t; }
-GemmTuning get_gemm_tuning() { return g_tuning; }
-
-int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
-  if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kSlabK)
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kSlabK);
-  if (a.symmetric && a.M != a.N) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric product needs M == N");
-  if (a.skip_c && (a.symmetric || !a.CT)) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: skip_c needs a transposed output and a general product");
-  if (!a.P || !a.Q || !a.C) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: null operand");
-  if (a.ldp < a.K || a.ldq < a.K || a.ldc < a.N || (a.D && a.ldd < a.N) || (a.CT && a.ldct < a.M))
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: leading dimension smaller than the row length");
-  if ((a.ldp | a.ldq) % 8 || (reinterpret_cast<uintptr_t>(a.P) | reinterpret_cast<uintptr_t>(a.Q)) % 16)
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: operands must be 16-byte aligned with leading dimensions multiple of 8");
-  if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
-      (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
-  int variant = a.symmetric ? g_tuning.symmetric_variant : g_tuning.general_variant;
+// Which tiling a product runs with: 1 = 256 x 256, 2 = 128 x 128.
+int choose_variant(const GemmNtArgs& a, const GemmTuning& tuning) {
+  int variant = a.symmetric ? tuning.symmetric_variant : tuning.general_variant;
   if (a.symmetric && variant == 3) {
     // The triangle of a symmetric product rarely tiles the machine evenly.  Compare the two tilings in rounds of
     // resident workgroups, the last partial round counting 1/splits (plus the partial-tile traffic, which grows with
@@ -526,7 +549,7 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
       const int rem = tiles % slots;
       double r = tiles / slots;
       if (rem != 0) {
-        const int splits = g_tuning.split_remainder ? std::min({slots / rem, a.K / kSlabK, g_tuning.max_splits}) : 1;
+        const int splits = tuning.split_remainder ? std::min({slots / rem, a.K / kSlabK, tuning.max_splits}) : 1;
         r += splits > 1 ? 1.0 / splits + 0.02 * splits : 1.0;
       }
       return r;
@@ -534,11 +557,42 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
     const int big = a.M / 256, big_tiles = big * (big + 1) / 2;
     variant = (4 * big_tiles >= 3 * device_cu_count() && rounds(256, 1) <= 0.6 * rounds(128, 2)) ? 1 : 2;
   }
+  return variant;
+}
+
+}  // namespace
+
+void set_gemm_tuning(const GemmTuning& t) {
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  g_tuning = t;
+}
+GemmTuning get_gemm_tuning() { return tuning_snapshot(); }
+
+int64_t gemm_nt_executed_flops(const GemmNtArgs& a) {
+  const GemmTuning tuning = tuning_snapshot();
+  const int tile = choose_variant(a, tuning) == 2 ? 128 : 256;
+  return 2 * static_cast<int64_t>(tile) * tile * a.K * tile_count(a, tile, tile);
+}
+
+int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0 || a.K <= 0 || a.M % 256 || a.N % 256 || a.K % kSlabK)
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: M=%d N=%d must be multiples of 256 and K=%d of %d", a.M, a.N, a.K, kSlabK);
+  if (a.symmetric && a.M != a.N) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: symmetric product needs M == N");
+  if (a.skip_c && (a.symmetric || !a.CT)) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: skip_c needs a transposed output and a general product");
+  if (!a.P || !a.Q || !a.C) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: null operand");
+  if (a.ldp < a.K || a.ldq < a.K || a.ldc < a.N || (a.D && a.ldd < a.N) || (a.CT && a.ldct < a.M))
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: leading dimension smaller than the row length");
+  if ((a.ldp | a.ldq) % 8 || (reinterpret_cast<uintptr_t>(a.P) | reinterpret_cast<uintptr_t>(a.Q)) % 16)
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: operands must be 16-byte aligned with leading dimensions multiple of 8");
+  if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
+      (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
+  const GemmTuning tuning = tuning_snapshot();
   // Slabs of 32 (three to five deep) were measured too: each slab row is then half a 128-byte line, the vector
   // cache looks every line up twice, and the products run 15-25 % slower than with slabs of 64 two deep.
-  if (variant == 2)  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
-    return launch<128, 128, 2, 2, 64, 2, 2>(a, scratch, stream);
-  return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, stream);  // 256x256 tile, 8 waves of 128x64, one workgroup per CU
+  if (choose_variant(a, tuning) == 2)  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
+    return launch<128, 128, 2, 2, 64, 2, 2>(a, scratch, tuning, stream);
+  return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, tuning, stream);  // 256x256 tile, 8 waves of 128x64, one workgroup per CU
 }
 
 }  // namespace mfsdp
