@@ -38,6 +38,9 @@ extern "C" {
 #define MFSDP_BF16 1
 #define MFSDP_F16 2 /* mfsdp_accumulate only */
 
+/* flag of mfsdp_muon_step_ex / mfsdp_muon_executed_flops */
+#define MFSDP_MUON_SHARED_MACHINE 1
+
 /* conversion a segment program applies while copying */
 #define MFSDP_CONVERT_NONE 0         /* raw element move, any elem_bytes */
 #define MFSDP_CONVERT_BF16_TO_F32 1  /* exact widening (Tensor.to(float32)) */
@@ -233,10 +236,10 @@ int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols);
 
 /*
  * Flops the Newton-Schulz kernels execute for `steps` iterations on a rows x cols matrix with the current tuning
- * (operands zero-padded to multiples of 256; the two symmetric products of a step compute only the tiles on or below
+ * and the flags of mfsdp_muon_step_ex (operands zero-padded to multiples of 256; the two symmetric products of a step compute only the tiles on or below
  * the diagonal).  The reference executes full products: steps * (4 m^2 n + 2 m^3) with m the short side.
  */
-int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps);
+int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps, int flags);
 
 /*
  * Quintic Newton-Schulz orthogonalisation of one matrix, the arithmetic of
@@ -265,13 +268,25 @@ int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype
                     float a, float b, float c, int steps, float eps, double adjusted_lr,
                     void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * mfsdp_muon_step with flags.  MFSDP_MUON_SHARED_MACHINE: the caller updates other matrices at the same time on
+ * other streams (each with its own workspace; a rank's whole matrices are independent of each other,
+ * torch/optim/_muon.py:285-318 loops over them).  The symmetric products X X^T and A A then take the tile shape that
+ * is best when the CUs they leave idle work for the other streams.  Results do not depend on the flag beyond the
+ * summation order inside a product.
+ */
+int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols,
+                       double lr, double weight_decay, double momentum, int nesterov,
+                       float a, float b, float c, int steps, float eps, double adjusted_lr, int flags,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Kernel selection for experiments (values <= 0 keep the current setting):
  * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
  * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU; for the symmetric products also 3, the default:
- * whichever of the two fills the CUs better for the size at hand), a reserved argument (slabs always stream
- * HBM -> LDS directly), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
+ * whichever of the two fills the CUs better for the size at hand), the tile rows the general products walk together
+ * (default 4), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
  * stagger >= 0 sets the K-walk start offset, in 64-element slabs, between consecutive tiles. */
-void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,
+void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder,
                            int max_splits, int stagger);
 
 /* ------------------------------------------------------------------ AdamW */

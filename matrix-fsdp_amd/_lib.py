@@ -21,7 +21,8 @@ CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
 DT_F16 = 2  # mfsdp_accumulate only
-ABI_VERSION = 3
+ABI_VERSION = 4
+MUON_SHARED_MACHINE = 1
 NOALLOC_MAX_SEGMENTS = 131071  # MFSDP_NOALLOC_MAX_SEGMENTS
 
 
@@ -72,7 +73,7 @@ SIGNATURES = {
     "mfsdp_hbm_probe": (c_int, [c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "mfsdp_cast": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mfsdp_muon_workspace_bytes": (c_int64, [c_int64, c_int64]),
-    "mfsdp_muon_executed_flops": (c_int64, [c_int64, c_int64, c_int]),
+    "mfsdp_muon_executed_flops": (c_int64, [c_int64, c_int64, c_int, c_int]),
     "mfsdp_newton_schulz": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_float, c_float, c_float, c_int, c_float, c_void_p, c_void_p, c_int64, c_void_p],
@@ -81,6 +82,11 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_double, c_double, c_double, c_int,
          c_float, c_float, c_float, c_int, c_float, c_double, c_void_p, c_int64, c_void_p],
+    ),
+    "mfsdp_muon_step_ex": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_double, c_double, c_double, c_int,
+         c_float, c_float, c_float, c_int, c_float, c_double, c_int, c_void_p, c_int64, c_void_p],
     ),
     "mfsdp_set_muon_tuning": (None, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "mfsdp_accumulate": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),

@@ -65,7 +65,7 @@ bool plan_workspace(int64_t rows, int64_t cols, void* base, Workspace* w) {
 // Newton-Schulz on the update already sitting in w.xraw (rows x cols bf16) with per-block sums of squares in
 // w.partials.  Leaves O in param layout at *ortho with leading dimension *ldo.
 int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, float a, float b, float c, int steps,
-                      float eps, const uint16_t** ortho, int* ldo, hipStream_t stream) {
+                      float eps, bool shared, const uint16_t** ortho, int* ldo, hipStream_t stream) {
   if (int rc = muon_norm(w.partials, n_partials, eps, w.scalars, stream)) return rc;
   // the input is rows x cols; the iteration wants the short side first
   uint16_t* same = w.tall ? w.XT[0] : w.X[0];   // rows_pad x cols_pad
@@ -79,13 +79,13 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     g.P = w.X[cur]; g.Q = w.X[cur]; g.D = nullptr; g.C = w.A; g.CT = nullptr;
     g.M = w.mp; g.N = w.mp; g.K = w.np;
     g.ldp = w.np; g.ldq = w.np; g.ldd = 0; g.ldc = w.mp; g.ldct = 0;
-    g.alpha = 1.0f; g.beta = 0.0f; g.symmetric = 1;
+    g.alpha = 1.0f; g.beta = 0.0f; g.symmetric = 1; g.shared = shared;
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.A; g.Q = w.A; g.D = w.A; g.C = w.B; g.CT = nullptr;
     g.M = w.mp; g.N = w.mp; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.mp; g.ldc = w.mp; g.ldct = 0;
-    g.alpha = c; g.beta = b; g.symmetric = 1;
+    g.alpha = c; g.beta = b; g.symmetric = 1; g.shared = shared;
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.B; g.Q = w.XT[cur]; g.D = w.X[cur]; g.C = w.X[nxt]; g.CT = w.XT[nxt];
@@ -126,12 +126,13 @@ extern "C" int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols) {
   return plan_workspace(rows, cols, nullptr, &w) ? w.bytes : 0;
 }
 
-extern "C" int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps) {
+extern "C" int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps, int flags) {
   Workspace w;
   if (steps < 0 || !plan_workspace(rows, cols, nullptr, &w)) return 0;
   GemmNtArgs gram{}, poly{}, update{};
   gram.M = gram.N = w.mp; gram.K = w.np; gram.symmetric = 1;
   poly.M = poly.N = poly.K = w.mp; poly.symmetric = 1;
+  gram.shared = poly.shared = (flags & MFSDP_MUON_SHARED_MACHINE) != 0;
   update.M = w.mp; update.N = w.np; update.K = w.mp;
   return steps * (gemm_nt_executed_flops(gram) + gemm_nt_executed_flops(poly) + gemm_nt_executed_flops(update));
 }
@@ -147,13 +148,13 @@ extern "C" int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t
   if (int rc = muon_momentum(update, nullptr, update_dtype, rows * cols, 0.0, 0, false, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
-  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, &ortho, &ldo, s)) return rc;
+  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, false, &ortho, &ldo, s)) return rc;
   return muon_extract(out_bf16, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, s);
 }
 
-extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, double lr,
-                               double weight_decay, double momentum, int nesterov, float a, float b, float c, int steps, float eps,
-                               double adjusted_lr, void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, double lr,
+                                  double weight_decay, double momentum, int nesterov, float a, float b, float c, int steps, float eps,
+                                  double adjusted_lr, int flags, void* workspace, int64_t workspace_bytes, void* stream) {
   Workspace w;
   if (int rc = check_common(rows, cols, steps, workspace, workspace_bytes, &w)) return rc;
   if (dtype != MFSDP_F32 && dtype != MFSDP_BF16) return fail(MFSDP_ERR_INVALID, "dtype must be f32 or bf16");
@@ -161,24 +162,34 @@ extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf
   if (!(lr >= 0.0)) return fail(MFSDP_ERR_INVALID, "Learning rate should be >= 0 but is: %g", lr);
   if (!(momentum >= 0.0)) return fail(MFSDP_ERR_INVALID, "momentum should be >= 0 but is: %g", momentum);
   if (!(weight_decay >= 0.0)) return fail(MFSDP_ERR_INVALID, "weight decay should be >= 0 but is: %g", weight_decay);
+  if (flags & ~MFSDP_MUON_SHARED_MACHINE) return fail(MFSDP_ERR_INVALID, "unknown flags 0x%x", flags);
   hipStream_t s = as_stream(stream);
   int n_partials = 0;
   if (int rc = muon_momentum(grad, momentum_buf, dtype, rows * cols, momentum, nesterov, true, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
-  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, &ortho, &ldo, s)) return rc;
+  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps,
+                                 (flags & MFSDP_MUON_SHARED_MACHINE) != 0, &ortho, &ldo, s))
+    return rc;
   // the host scalars are doubles, as in Python: 1 - lr * wd and -adjusted_lr are rounded to fp32 once, where the
   // tensor operation takes them
   const float decay = static_cast<float>(1.0 - lr * weight_decay);
   return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, decay, static_cast<float>(-adjusted_lr), s);
 }
 
-extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int direct_to_lds, int split_remainder,
+extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, double lr,
+                               double weight_decay, double momentum, int nesterov, float a, float b, float c, int steps, float eps,
+                               double adjusted_lr, void* workspace, int64_t workspace_bytes, void* stream) {
+  return mfsdp_muon_step_ex(param, grad, momentum_buf, dtype, rows, cols, lr, weight_decay, momentum, nesterov, a, b, c, steps, eps,
+                            adjusted_lr, 0, workspace, workspace_bytes, stream);
+}
+
+extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder,
                                       int max_splits, int stagger) {
   GemmTuning t = get_gemm_tuning();
   if (general_variant > 0) t.general_variant = general_variant;
   if (symmetric_variant > 0) t.symmetric_variant = symmetric_variant;
-  if (direct_to_lds > 0) t.direct_to_lds = direct_to_lds == 1;
+  if (group_m > 0) t.group_m = group_m;
   if (split_remainder > 0) t.split_remainder = split_remainder == 1;
   if (max_splits > 0) t.max_splits = max_splits;
   if (stagger >= 0) t.stagger = stagger;

@@ -24,6 +24,8 @@ struct GemmNtArgs {
   float alpha, beta;
   int symmetric;
   int skip_c;  // general product with CT set: write only the transposed output
+  int shared;  // other matrices' products run beside this one on other streams: a symmetric product then takes the
+               // 256 x 256 tiles even where their triangle fills only part of the CUs (the rest works for the others)
 };
 
 // Device scratch for the K-split pieces of the last partial round of tiles (fp32 partial tiles).
@@ -36,7 +38,7 @@ constexpr int64_t kGemmPartialsBytes = 64ll << 20;
 struct GemmTuning {
   int general_variant = 1;    // 1: 256x256 tile / 8 waves / one workgroup per CU, 2: 128x128 tile / 4 waves / two per CU
   int symmetric_variant = 3;  // 1, 2 as above; 3: whichever fills the CUs better for the product at hand
-  int direct_to_lds = 1;      // reserved (slabs always stream HBM -> LDS directly)
+  int group_m = 4;            // general products: tile rows walked together (the workgroups of one XCD share their P panels)
   int split_remainder = 1;    // split the tiles of the last partial round along K
   int max_splits = 16;
   int stagger = 0;            // K-walk start offset (slabs) between consecutive tiles; 0 = none

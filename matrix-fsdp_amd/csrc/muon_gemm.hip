@@ -11,7 +11,7 @@
 // current one feeds the MFMAs.
 //
 // Tile scheduling.  Tiles are handed to workgroups so that the groups sharing an XCD (block ids
-// congruent mod 8) work on neighbouring tiles and reuse that XCD's L2.  When the tile count is not a
+// congruent mod 8) work on neighbouring tiles and reuse that XCD's L2, whatever the tile count.  When the tile count is not a
 // multiple of the number of resident workgroups, the tiles of the last, partial round are split along
 // K into pieces that fill the machine once more for a fraction of a tile's time; each piece leaves an
 // fp32 partial tile in a workspace and a small fix-up kernel sums the pieces in split order and runs
@@ -50,11 +50,11 @@ struct Schedule {
   int splits;       // K pieces per remaining tile (block ids from full_tiles on); 1 when nothing remains
   float* partials;  // [remaining tiles][splits][BM][BN] fp32
   int stagger;      // tile t starts its K walk (t * stagger) slabs in and wraps around; 0 = every tile starts at slab 0
+  int group_m;      // tile rows per group of the general products' tile order
 };
 
 // logical tile index -> (tm, tn)
-template <int GROUP_M>
-__device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_n, bool symmetric, int* tm, int* tn) {
+__device__ __forceinline__ void tile_coords(int group_m, int logical, int tiles_m, int tiles_n, bool symmetric, int* tm, int* tn) {
   if (symmetric) {
     // the lower triangle row by row: t = i(i+1)/2 + j, j <= i
     int i = static_cast<int>((__fsqrt_rn(8.0f * static_cast<float>(logical) + 1.0f) - 1.0f) * 0.5f);
@@ -64,11 +64,11 @@ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_
     *tn = logical - i * (i + 1) / 2;
     return;
   }
-  // GROUP_M tile rows at a time, walking down the rows before moving to the next tile column
-  const int per_group = GROUP_M * tiles_n;
+  // group_m tile rows at a time, walking down the rows before moving to the next tile column
+  const int per_group = group_m * tiles_n;
   const int group = logical / per_group;
-  const int first_m = group * GROUP_M;
-  const int rows = min(GROUP_M, tiles_m - first_m);
+  const int first_m = group * group_m;
+  const int rows = min(group_m, tiles_m - first_m);
   const int in_group = logical - group * per_group;
   *tm = first_m + in_group % rows;
   *tn = in_group / rows;
@@ -102,8 +102,10 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   const bool whole = block < sched.full_tiles;
   int logical, split = 0, piece_tile = 0;
   if (whole) {
-    logical = block;
-    if (sched.full_tiles % kXcds == 0) logical = (block % kXcds) * (sched.full_tiles / kXcds) + block / kXcds;
+    // workgroup ids congruent mod 8 run on one XCD: hand each XCD one contiguous eighth of the tile order (the first
+    // full_tiles % 8 of them one tile more), so that the workgroups sharing an L2 work on neighbouring tiles
+    const int xcd = block % kXcds, each = sched.full_tiles / kXcds, extra = sched.full_tiles % kXcds;
+    logical = xcd * each + (xcd < extra ? xcd : extra) + block / kXcds;
   } else {
     const int piece = block - sched.full_tiles;
     piece_tile = piece / sched.splits;
@@ -111,7 +113,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     logical = sched.full_tiles + piece_tile;
   }
   int tm, tn;
-  tile_coords<4>(logical, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
+  tile_coords(sched.group_m, logical, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
   const int row0 = tm * BM;
   const int col0 = tn * BN;
   const int k_slabs_total = a.K / BK;
@@ -406,7 +408,7 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
   const int sub = blockIdx.x % kSubsPerTile;
   const int sub_row0 = (sub / (BN / kSub)) * kSub, sub_col0 = (sub % (BN / kSub)) * kSub;
   int tm, tn;
-  tile_coords<4>(sched.full_tiles + tile, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
+  tile_coords(sched.group_m, sched.full_tiles + tile, sched.tiles_m, sched.tiles_n, a.symmetric != 0, &tm, &tn);
   const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
   uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
@@ -492,6 +494,7 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, const GemmTuning& tu
   s.splits = 1;
   s.partials = static_cast<float*>(scratch.partials);
   s.stagger = tuning.stagger;
+  s.group_m = std::max(1, tuning.group_m);
   const int rem = tiles % slots;
   if (tuning.split_remainder && rem != 0 && scratch.partials != nullptr) {
     // fill the machine once more with pieces of the leftover tiles; cap the pieces per tile so that the summing stays short
@@ -556,6 +559,10 @@ int choose_variant(const GemmNtArgs& a, const GemmTuning& tuning) {
     };
     const int big = a.M / 256, big_tiles = big * (big + 1) / 2;
     variant = (4 * big_tiles >= 3 * device_cu_count() && rounds(256, 1) <= 0.6 * rounds(128, 2)) ? 1 : 2;
+    // On a machine shared with other matrices' kernels the CUs a part-filling triangle of big tiles leaves idle are
+    // not lost, and a big tile moves fewer LDS bytes per flop: three hidden4096 matrices on three streams take 7.97 ms
+    // with big tiles against 8.73 ms with small ones (8.47 ms one after the other).
+    if (a.shared && 4 * big_tiles >= device_cu_count()) variant = 1;
   }
   return variant;
 }

@@ -5,7 +5,8 @@ per-parameter state (``momentum_buffer = zeros_like(grad)``) follow
 torch/optim/_muon.py:87-202, which is the optimizer the reference
 instantiates for owner-rank matrices (matrix_fsdp/optim/wrapper.py:416-429).
 ``step()`` runs momentum, Newton-Schulz and the parameter update of every
-matrix through ``mfsdp_muon_step``; nothing falls back to torch arithmetic.
+matrix through ``mfsdp_muon_step_ex`` (independent matrices side by side where
+that pays); nothing falls back to torch arithmetic.
 """
 from __future__ import annotations
 
@@ -45,6 +46,7 @@ class Muon(torch.optim.Muon):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        jobs = []
         for group in self.param_groups:
             for p in group["params"]:
                 if p.grad is None:
@@ -59,14 +61,8 @@ class Muon(torch.optim.Muon):
                 state = self.state[p]
                 if "momentum_buffer" not in state:
                     state["momentum_buffer"] = torch.zeros_like(grad, memory_format=torch.preserve_format)
-                if self._workspace is None or self._workspace.device != p.device:
-                    self._workspace = F.MuonWorkspace(p.device)
-                lr = group["lr"]
-                F.muon_step(
-                    p.data,
-                    grad.contiguous(),
-                    state["momentum_buffer"],
-                    lr=float(lr),
+                keywords = dict(
+                    lr=float(group["lr"]),
                     weight_decay=group["weight_decay"],
                     momentum=group["momentum"],
                     nesterov=group["nesterov"],
@@ -74,6 +70,14 @@ class Muon(torch.optim.Muon):
                     ns_steps=group["ns_steps"],
                     eps=group["eps"],
                     adjust_lr_fn=group["adjust_lr_fn"],
-                    workspace=self._workspace,
                 )
+                jobs.append((p.data, grad.contiguous(), state["momentum_buffer"], keywords))
+        # the matrices are independent: one device's share goes to muon_step_many, which runs small ones side by side
+        by_device: dict[torch.device, list] = {}
+        for job in jobs:
+            by_device.setdefault(job[0].device, []).append(job)
+        for device, device_jobs in by_device.items():
+            if self._workspace is None or self._workspace.device != device:
+                self._workspace = F.MuonWorkspace(device)
+            F.muon_step_many(device_jobs, workspace=self._workspace)
         return loss

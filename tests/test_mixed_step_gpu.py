@@ -179,6 +179,35 @@ def test_muon_step_full_size_parameter_delta(shape):
     assert torch.allclose(buf_dev.cpu(), buf_torch_gpu, rtol=1e-6, atol=1e-9)
 
 
+def test_hidden4096_matrices_side_by_side_against_torch_muon():
+    """The three matrices of a hidden4096 layer updated at the same time on side streams (their symmetric products then
+    run on 256 x 256 tiles): every parameter delta against ``torch.optim.Muon.step`` on this GPU and, for the square
+    one, against the CPU oracle."""
+    torch.set_num_threads(16)
+    shapes = [(4096, 4096), (12288, 4096), (11008, 4096)]
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    p0 = [normal_flat(r * c, 0.02, 51 + i, torch.float32).view(r, c) for i, (r, c) in enumerate(shapes)]
+    grads = [normal_flat(r * c, 1e-3, 61 + i, torch.bfloat16).float().view(r, c) for i, (r, c) in enumerate(shapes)]
+    buf0 = [normal_flat(r * c, 1e-3, 71 + i, torch.float32).view(r, c) for i, (r, c) in enumerate(shapes)]
+    p_dev, b_dev = [p.to(DEV) for p in p0], [b.to(DEV) for b in buf0]
+    F.muon_step_many([(p_dev[i], grads[i].to(DEV), b_dev[i], kw) for i in range(3)])
+    torch_params = [torch.nn.Parameter(p.to(DEV)) for p in p0]
+    opt = torch.optim.Muon(torch_params, **kw)
+    for tp, g, b in zip(torch_params, grads, buf0):
+        opt.state[tp]["momentum_buffer"] = b.to(DEV)
+        tp.grad = g.to(DEV)
+    opt.step()
+    for i, shape in enumerate(shapes):
+        delta = p_dev[i].cpu() - p0[i]
+        to_torch_gpu = rel_fro(delta, torch_params[i].detach().cpu() - p0[i])
+        _report({"test": "muon_step_many_delta", "shape": list(shape), "vs_torch_gpu": to_torch_gpu})
+        assert to_torch_gpu < MUON_TOL, (shape, to_torch_gpu)
+        assert torch.allclose(b_dev[i].cpu(), opt.state[torch_params[i]]["momentum_buffer"].cpu(), rtol=1e-6, atol=1e-9)
+    p_ref, b_ref = p0[0].clone(), buf0[0].clone()
+    OO.muon_step(p_ref, grads[0], b_ref, **kw)
+    assert rel_fro(p_dev[0].cpu() - p0[0], p_ref - p0[0]) < MUON_TOL
+
+
 @pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("shape", [(512, 768), (768, 512), (1024, 1024)])
 def test_symmetric_tile_variants_forced(shape, variant):

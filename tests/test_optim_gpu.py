@@ -103,6 +103,35 @@ def test_muon_step_matches_torch_optim_muon_on_device_inputs():
     assert torch.allclose(buf.cpu(), opt.state[p_ref]["momentum_buffer"], rtol=1e-6, atol=1e-9)
 
 
+def test_muon_step_many_matches_one_matrix_at_a_time():
+    """Independent matrices spread over side streams: the same bits as one call per matrix on the calling stream (for
+    matrices this small the flag does not change the tiling), work enqueued afterwards sees the updates, and an
+    optimizer over several parameter groups goes the same way."""
+    shapes = [(512, 768), (768, 512), (256, 256), (320, 200), (1024, 512)]
+    hypers = [dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True), dict(lr=0.01, weight_decay=0.0, momentum=0.9, nesterov=False, adjust_lr_fn="match_rms_adamw")]
+    params = [make(sh, 100 + i, 0.02) for i, sh in enumerate(shapes)]
+    grads = [make(sh, 200 + i).bfloat16().float() for i, sh in enumerate(shapes)]
+    bufs = [make(sh, 300 + i) for i, sh in enumerate(shapes)]
+    one_p, one_b = [p.to(DEV) for p in params], [b.to(DEV) for b in bufs]
+    ws = F.MuonWorkspace(DEV)
+    for i in range(len(shapes)):
+        F.muon_step(one_p[i], grads[i].to(DEV), one_b[i], workspace=ws, **hypers[i % 2])
+    many_p, many_b = [p.to(DEV) for p in params], [b.to(DEV) for b in bufs]
+    dev_grads = [g.to(DEV) for g in grads]
+    F.muon_step_many([(many_p[i], dev_grads[i], many_b[i], hypers[i % 2]) for i in range(len(shapes))])
+    total = sum(p.sum() for p in many_p)  # enqueued on the calling stream right behind the batch
+    for i in range(len(shapes)):
+        assert torch.equal(many_p[i], one_p[i]) and torch.equal(many_b[i], one_b[i])
+        p_ref, b_ref = params[i].clone(), bufs[i].clone()
+        O.muon_step(p_ref, grads[i], b_ref, **hypers[i % 2])
+        assert rel_fro(many_p[i].cpu() - params[i], p_ref - params[i]) < MUON_TOL
+    assert float(total) == float(sum(p.sum() for p in one_p))
+    F.muon_step_many([])
+    F.muon_step_many([(many_p[0], dev_grads[0], many_b[0], hypers[0])])  # a single matrix stays on the calling stream
+    F.muon_step(one_p[0], dev_grads[0], one_b[0], workspace=ws, **hypers[0])
+    assert torch.equal(many_p[0], one_p[0])
+
+
 def test_muon_argument_errors():
     p = torch.zeros(8, 8, device=DEV)
     with pytest.raises(ValueError, match="2D"):
