@@ -35,7 +35,7 @@ HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 NS_COEFFS = (3.4445, -4.7750, 2.0315)
 # figures taken from the committed rocprofv3 counter profiles (they cannot be measured from inside this process)
-PROFILED_TRAFFIC = {"bytes_per_launch": 812_800_000, "source": "profiles/segment_program_hbm_traffic.md"}
+PROFILED_TRAFFIC = {"bytes_per_launch": 812_818_425, "source": "profiles/segment_program_hbm_traffic.md"}
 PROFILED_MUON = {
     # SQ_VALU_MFMA_BUSY_CYCLES over the SIMD cycles of the dispatch, per tile shape
     "mfma_busy": {"gemm_nt_kernel<256,256> (general products)": 0.524, "gemm_nt_kernel<128,128> (symmetric products)": 0.446},
