@@ -395,11 +395,12 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   }
 }
 
-// Sums the K pieces of every split tile in split order and applies the epilogue of gemm_nt_kernel.  A workgroup
-// finishes a 64 x 64 block of a tile: thread t owns four consecutive columns of rows t / 16, t / 16 + 16, ...; the
-// transposed / mirrored copy goes through LDS so that both orientations leave in whole 16-byte, row-contiguous stores.
+// Sums the K pieces of every split tile in split order and applies the epilogue of gemm_nt_kernel.  A workgroup of
+// 1024 threads finishes a 64 x 64 block of a tile, thread t four consecutive columns of row t / 16; the transposed /
+// mirrored copy goes through LDS so that both orientations leave in whole 16-byte, row-contiguous stores.
+constexpr int kFixupThreads = 1024;
 template <int BM, int BN>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kFixupThreads)
 splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kSub = 64;
   constexpr int kSubsPerTile = (BM / kSub) * (BN / kSub);
@@ -418,52 +419,45 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
     ldct = a.ldc;
   }
   const int t = threadIdx.x;
-  const int lcol = sub_col0 + (t % 16) * 4;
+  const int r = t / 16, c = (t % 16) * 4;  // position inside the 64 x 64 block
+  const int lrow = sub_row0 + r, lcol = sub_col0 + c;
+  const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
+  // four loads in flight at a time; the sum itself stays in split order
+  f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+  int s = 0;
+  for (; s + 4 <= sched.splits; s += 4) {
+    f32x4 piece[4];
 #pragma unroll
-  for (int rr = 0; rr < 4; ++rr) {
-    const int lrow = sub_row0 + rr * 16 + t / 16;
-    const float* base = sched.partials + static_cast<int64_t>(tile) * sched.splits * (BM * BN) + lrow * BN + lcol;
-    // four loads in flight at a time; the sum itself stays in split order
-    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-    int s = 0;
-    for (; s + 4 <= sched.splits; s += 4) {
-      f32x4 piece[4];
+    for (int u = 0; u < 4; ++u) piece[u] = *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s + u) * (BM * BN));
 #pragma unroll
-      for (int u = 0; u < 4; ++u) piece[u] = *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s + u) * (BM * BN));
-#pragma unroll
-      for (int u = 0; u < 4; ++u) sum += piece[u];
-    }
-    for (; s < sched.splits; ++s) sum += *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN));
-    const int row = tm * BM + lrow, col = tn * BN + lcol;
-    float v[4] = {a.alpha * sum.x, a.alpha * sum.y, a.alpha * sum.z, a.alpha * sum.w};
-    if (D != nullptr) {
-      const u32x2 d = *reinterpret_cast<const u32x2*>(D + static_cast<int64_t>(row) * a.ldd + col);
-      v[0] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x));
-      v[1] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x >> 16));
-      v[2] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y));
-      v[3] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y >> 16));
-    }
-    const uint32_t lo = pack_bf16x2(v[0], v[1]);
-    const uint32_t hi = pack_bf16x2(v[2], v[3]);
-    if (!a.skip_c) {
-      const u32x2 packed = {lo, hi};
-      *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
-    }
-    if (CT != nullptr) {
-      const int c = (t % 16) * 4, r = rr * 16 + t / 16;
-      transposed[c][r] = static_cast<uint16_t>(lo);
-      transposed[c + 1][r] = static_cast<uint16_t>(lo >> 16);
-      transposed[c + 2][r] = static_cast<uint16_t>(hi);
-      transposed[c + 3][r] = static_cast<uint16_t>(hi >> 16);
-    }
+    for (int u = 0; u < 4; ++u) sum += piece[u];
   }
-  if (CT == nullptr) return;
+  for (; s < sched.splits; ++s) sum += *reinterpret_cast<const f32x4*>(base + static_cast<int64_t>(s) * (BM * BN));
+  const int row = tm * BM + lrow, col = tn * BN + lcol;
+  float v[4] = {a.alpha * sum.x, a.alpha * sum.y, a.alpha * sum.z, a.alpha * sum.w};
+  if (D != nullptr) {
+    const u32x2 d = *reinterpret_cast<const u32x2*>(D + static_cast<int64_t>(row) * a.ldd + col);
+    v[0] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x));
+    v[1] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.x >> 16));
+    v[2] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y));
+    v[3] += a.beta * bf16_bits_to_float(static_cast<uint16_t>(d.y >> 16));
+  }
+  const uint32_t lo = pack_bf16x2(v[0], v[1]);
+  const uint32_t hi = pack_bf16x2(v[2], v[3]);
+  if (!a.skip_c) {
+    const u32x2 packed = {lo, hi};
+    *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
+  }
+  if (CT == nullptr) return;  // uniform over the workgroup
+  transposed[c][r] = static_cast<uint16_t>(lo);
+  transposed[c + 1][r] = static_cast<uint16_t>(lo >> 16);
+  transposed[c + 2][r] = static_cast<uint16_t>(hi);
+  transposed[c + 3][r] = static_cast<uint16_t>(hi >> 16);
   __syncthreads();
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int r = half * 32 + t / 8, chunk = t % 8;  // row of the transposed block = column of the tile
-    *reinterpret_cast<u32x4*>(CT + static_cast<int64_t>(tn * BN + sub_col0 + r) * ldct + tm * BM + sub_row0 + chunk * 8) =
-        *reinterpret_cast<const u32x4*>(&transposed[r][chunk * 8]);
+  if (t < kSub * 8) {
+    const int tr = t / 8, chunk = t % 8;  // row of the transposed block = column of the tile
+    *reinterpret_cast<u32x4*>(CT + static_cast<int64_t>(tn * BN + sub_col0 + tr) * ldct + tm * BM + sub_row0 + chunk * 8) =
+        *reinterpret_cast<const u32x4*>(&transposed[tr][chunk * 8]);
   }
 }
 
@@ -529,7 +523,7 @@ int launch(const GemmNtArgs& a, const GemmScratch& scratch, const GemmTuning& tu
   MFSDP_CHECK_LAUNCH("gemm_nt_kernel");
   if (s.splits > 1) {
     const int fix_blocks = (tiles - s.full_tiles) * (BM / 64) * (BN / 64);
-    hipLaunchKernelGGL((splitk_fixup_kernel<BM, BN>), dim3(fix_blocks), dim3(256), 0, stream, a, s);
+    hipLaunchKernelGGL((splitk_fixup_kernel<BM, BN>), dim3(fix_blocks), dim3(kFixupThreads), 0, stream, a, s);
     MFSDP_CHECK_LAUNCH("splitk_fixup_kernel");
   }
   return MFSDP_OK;
