@@ -23,13 +23,15 @@ FLAGS = [
     "-fPIC",
     "-Wall",
     "-Wno-unused-function",
-    # keep the compiler from emitting packed fp32 arithmetic
+    # keep the compiler from emitting packed fp32 arithmetic (v_pk_fma_f32 and friends).  A device-pass feature: the
+    # gfx950 pass honours it (tests/test_build_flags.py compiles a probe both ways), hipcc's host pass does not know it
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
 def _run(cmd: list[str]) -> None:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # the x86 host pass of every hipcc call prints this once per source for the device-only feature above
     noise = "'-packed-fp32-ops' is not a recognized feature for this target"
     out = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
     if proc.returncode != 0:
