@@ -2,7 +2,7 @@
 //
 // Both operands are K-contiguous (an "NT" product), which is what every Newton-Schulz product
 // reduces to once X and X^T are both kept: X X^T, A A^T (A symmetric) and B (X^T)^T.  A workgroup owns
-// a BM x BN tile of C; its waves each own a (BM/WM) x (BN/WN) sub-tile built from 32x32x16 bf16 MFMAs
+// a BM x BN tile of C; its waves each own a (BM/WM) x (BN/WN) sub-tile built from 16x16x32 bf16 MFMAs
 // with fp32 accumulators.  K is walked in slabs of BK (64 or 32): the slab of P and Q is staged in LDS as
 // rows of BK bf16 whose 16-byte chunks are XOR-swizzled with the row index: the LDS has 64 banks of 4
 // bytes, 256 / (2 BK) rows span them once, so any 16 consecutive rows read at one logical chunk touch every
@@ -28,7 +28,6 @@ namespace mfsdp {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -82,16 +81,17 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kWaves = WM * WN;
   constexpr int kWaveM = BM / WM;     // rows of C per wave
   constexpr int kWaveN = BN / WN;
-  constexpr int TM = kWaveM / 32;     // 32x32 MFMA tiles per wave
-  constexpr int TN = kWaveN / 32;
+  constexpr int TM = kWaveM / 16;     // 16x16 MFMA tiles per wave
+  constexpr int TN = kWaveN / 16;
+  constexpr int TMH = TM / 2;         // tile rows one half step covers
   constexpr int kChunks = BK / 8;               // 16-byte chunks per slab row (row = BK bf16)
   constexpr int kRowsPerSweep = 128 / BK;       // slab rows that together span the 64 LDS banks once (256 bytes)
   constexpr int kRowsPerLoad = 512 / BK;        // slab rows one wave-level 1 KiB load fills
-  constexpr int kSteps = BK / 16;               // k16 MFMA steps per slab
+  constexpr int kSteps = BK / 32;               // k32 MFMA steps per slab, each run as two half steps of TMH tile rows
   constexpr int kLoadsP = BM / kRowsPerLoad / kWaves, kLoadsQ = BN / kRowsPerLoad / kWaves;
   constexpr int kLoadsPerSlab = kLoadsP + kLoadsQ;  // direct-to-LDS loads one wave issues per slab
   static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0, "slab must divide over the waves");
-  static_assert(kSteps % 2 == 0 && STAGES >= 2 && (STAGES - 1) * kLoadsPerSlab < 64, "pipeline shape");
+  static_assert(kSteps % 2 == 0 && TM % 2 == 0 && STAGES >= 2 && (STAGES - 1) * kLoadsPerSlab < 64, "pipeline shape");
   constexpr int kStageElems = (BM + BN) * BK;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -169,40 +169,42 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int i = 0; i < kLoadsQ; ++i) load_q(k0, stage, i);
   };
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-  const int frag_row = lane & 31;   // row of the 32-row MFMA operand this lane supplies
-  const int frag_half = lane >> 5;  // which 8 of the 16 k values
+  // 16x16x32 MFMA operands: lane l supplies row l % 16 of its 16-row block and the 8 k values of chunk l / 16 of
+  // the 32 wide step.  (At equal peak rate this shape draws less power than 32x32x16 on operands with random
+  // bits, and under sustained load the chip's clock is set by power: measured 2.0 against 1.8 PFLOP/s for bare
+  // MFMA streams.)
+  const int frag_row = lane & 15;
+  const int frag_chunk = lane >> 4;
 
-  // LDS offsets of this lane's fragment chunk for the k16 steps of a slab (the row part of the swizzle only
-  // depends on frag_row, every 32-row block starts at a multiple of 16 rows)
+  // LDS offsets of this lane's fragment chunk for the k32 steps of a slab (the row part of the swizzle only
+  // depends on frag_row: every 16-row block starts at a multiple of 16 rows)
   const __bf16* frag_p = smem + (wave_m * kWaveM + frag_row) * BK;
   const __bf16* frag_q = smem + BM * BK + (wave_n * kWaveN + frag_row) * BK;
-  auto load_frags = [&](int stage, int kk, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
-    const int off = stage * kStageElems + (((kk * 2 + frag_half) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 32 * BK);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 32 * BK);
+  auto frag_off = [&](int stage, int kk) {
+    return stage * kStageElems + (((kk * 4 + frag_chunk) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
   };
   // Software pipeline.  STAGES slabs are resident or in flight: the slab being multiplied and the next
-  // STAGES - 1, streamed HBM -> LDS while the MFMAs run.  Fragments are double buffered in registers: the
-  // TM + TN 128-bit LDS reads of step kk+1 are issued before the MFMAs of step kk (and waited for BEFORE the
-  // reads of step kk+2 are issued, which costs nothing), so their latency hides behind TM*TN MFMAs.  The one
-  // barrier per slab sits before the slab's last k16 step: by then every wave has its last fragments of the
-  // current stage in registers (the stage can be refilled with the slab STAGES ahead) and its share of the next
-  // slab has landed, so the next slab's first fragments are fetched under this slab's last MFMAs.
+  // STAGES - 1, streamed HBM -> LDS while the MFMAs run.  A k32 step runs as two half steps of TMH x TN MFMAs
+  // (the upper and the lower tile rows of the wave).  Fragments: the Q side (all TN of a step) is double
+  // buffered, the P side holds one buffer per half; the first half of a step reads the P fragments of its second
+  // half, the second half reads the next step's Q fragments and first-half P fragments, so every 128-bit LDS read
+  // has half a step of MFMAs to come back (it is waited for at the start of the next half step).  The one barrier
+  // per slab sits before the slab's last half step: by then every wave has its last fragments of the current
+  // stage in registers (the stage can be refilled with the slab STAGES ahead) and its share of the next slab has
+  // landed, so the next slab's first fragments are fetched under this slab's last MFMAs.
   constexpr int kWaitLds = 0xC07F;  // s_waitcnt lgkmcnt(0), vmcnt / expcnt fields at their maxima
   // s_waitcnt lgkmcnt(0) vmcnt(N): loads return in order, so this leaves the N most recent ones in flight
   constexpr int kInFlight = (STAGES - 2) * kLoadsPerSlab;
   constexpr int kWaitNextSlab = 0x0070 | (kInFlight & 0xF) | ((kInFlight >> 4) << 14);
-  bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+  bf16x8 fa_lo[TMH], fa_hi[TMH], fb0[TN], fb1[TN];
   // Loads are issued unconditionally, for a slab number clamped to the last one: past the end of the walk they
   // fetch the last slab once more into a stage nobody reads again.  (A branch around a load in the middle of the
   // MFMAs makes the register allocator spill the accumulators.)
@@ -216,43 +218,37 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     constexpr int kAfterFirst = (STAGES - 2) * kLoadsPerSlab + kLoadsP;
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kAfterFirst & 0xF) | ((kAfterFirst >> 4) << 14));
     __syncthreads();
-    load_frags(0, 0, fa0, fb0);
+    const int off = frag_off(0, 0);
+#pragma unroll
+    for (int i = 0; i < TMH; ++i) fa_lo[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 16 * BK);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb0[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 16 * BK);
   }
-  // One k16 step: the MFMAs on the fragments in hand (use_a, use_b), the LDS reads of the fragments after them
-  // (stage / kk -> next_a, next_b) and kLoads slab loads, interleaved instruction by instruction: MFMA, LDS read,
-  // MFMA, LDS read, slab load, ...  The matrix pipe is handed to the oldest wave that has an MFMA ready, so
-  // whenever one of the two waves of a SIMD sits at the barrier the other runs alone, and then every clump of
-  // other instructions between two MFMAs is a bubble in the pipe.
-  auto step = [&](const bf16x8 (&use_a)[TM], const bf16x8 (&use_b)[TN], bf16x8 (&next_a)[TM], bf16x8 (&next_b)[TN],
-                  int read_stage, int read_kk, auto loads_tag, auto&& load) {
+  // One half step: the TMH x TN MFMAs on the fragments in hand (use_a for tile rows row0.., use_b), kReads LDS
+  // reads (read(r), one behind each of the first MFMAs) and kLoads slab loads, interleaved instruction by
+  // instruction: MFMA, LDS read, MFMA, LDS read, ..., slab load, ...  The matrix pipe is handed to the oldest wave
+  // that has an MFMA ready, so whenever one of the two waves of a SIMD sits at the barrier the other runs alone,
+  // and then every clump of other instructions between two MFMAs is a bubble in the pipe.
+  auto half_step = [&](auto row0_tag, const bf16x8 (&use_a)[TMH], const bf16x8 (&use_b)[TN], auto reads_tag, auto&& read,
+                       auto loads_tag, auto&& load) {
+    constexpr int kRow0 = decltype(row0_tag)::value;
+    constexpr int kReads = decltype(reads_tag)::value;
     constexpr int kLoads = decltype(loads_tag)::value;
-    constexpr int kMfma = TM * TN, kReads = TM + TN;
+    constexpr int kMfma = TMH * TN;
     constexpr int kChunks_ = kLoads > 0 ? kLoads : 1;
     constexpr int kPer = kMfma / kChunks_;
-    constexpr int kReadsPerMfma = 2;
-    static_assert(kMfma % kChunks_ == 0 && kReads <= kReadsPerMfma * kMfma, "step shape");
-    const int off = read_stage * kStageElems + (((read_kk * 2 + frag_half) ^ ((frag_row / kRowsPerSweep) % kChunks)) << 3);
+    static_assert(kMfma % kChunks_ == 0 && kReads <= kMfma, "half step shape");
 #pragma unroll
     for (int c = 0; c < kChunks_; ++c) {
 #pragma unroll
       for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
-        // Q fragments first: the MFMAs walk the tile row by row, so the first of them need every Q fragment but
-        // only the first P fragment.  Two reads go out behind each of the first MFMAs, so that the last one has
-        // the rest of the step to come back.
-#pragma unroll
-        for (int r = kReadsPerMfma * n; r < kReadsPerMfma * (n + 1) && r < kReads; ++r) {
-          if (r < TN) next_b[r] = *reinterpret_cast<const bf16x8*>(frag_q + off + r * 32 * BK);
-          else next_a[r - TN] = *reinterpret_cast<const bf16x8*>(frag_p + off + (r - TN) * 32 * BK);
-        }
-        acc[n / TN][n % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use_a[n / TN], use_b[n % TN], acc[n / TN][n % TN], 0, 0, 0);
+        if (n < kReads) read(n);
+        acc[kRow0 + n / TN][n % TN] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(use_a[n / TN], use_b[n % TN], acc[kRow0 + n / TN][n % TN], 0, 0, 0);
       }
 #pragma unroll
       for (int n = c * kPer; n < (c + 1) * kPer; ++n) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-        constexpr int kNone = 0;
-        const int reads = kReadsPerMfma * (n + 1) <= kReads ? kReadsPerMfma : (kReadsPerMfma * n < kReads ? kReads - kReadsPerMfma * n : kNone);
-        if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        else if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (n < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
       }
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kLoads > 0) {
@@ -260,6 +256,25 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+  using Zero = std::integral_constant<int, 0>;
+  using Upper = std::integral_constant<int, TMH>;
+  // first half of step kk (fragments in fa_lo / use_b): reads the second half's P fragments
+  auto first_half = [&](const bf16x8 (&use_b)[TN], int read_stage, int kk, auto loads_tag, auto&& load) {
+    const int off = frag_off(read_stage, kk);
+    half_step(Zero{}, fa_lo, use_b, std::integral_constant<int, TMH>{},
+              [&](int r) { fa_hi[r] = *reinterpret_cast<const bf16x8*>(frag_p + off + (TMH + r) * 16 * BK); }, loads_tag, load);
+  };
+  // second half (fa_hi / use_b): reads the Q fragments and the first-half P fragments of the step after it
+  auto second_half = [&](const bf16x8 (&use_b)[TN], bf16x8 (&next_b)[TN], int read_stage, int read_kk, auto loads_tag, auto&& load) {
+    const int off = frag_off(read_stage, read_kk);
+    half_step(Upper{}, fa_hi, use_b, std::integral_constant<int, TN + TMH>{},
+              [&](int r) {
+                // Q fragments first: the next step's first MFMAs need every one of them but only the first P fragment
+                if (r < TN) next_b[r] = *reinterpret_cast<const bf16x8*>(frag_q + off + r * 16 * BK);
+                else fa_lo[r - TN] = *reinterpret_cast<const bf16x8*>(frag_p + off + (r - TN) * 16 * BK);
+              },
+              loads_tag, load);
   };
   int stage = 0;
   for (int it = 0; it < n_slabs; ++it) {
@@ -272,22 +287,28 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       if (kk == 0) {
         // second half of the refill of the stage the previous slab's barrier released (its P rows went out there)
         const int k0 = k0_clamped(it - 1 + STAGES);
-        step(fa0, fb0, fa1, fb1, stage, kk + 1, std::integral_constant<int, kLoadsQ>{}, [&](int l) { load_q(k0, prev_stage, l); });
+        first_half(fb0, stage, kk, std::integral_constant<int, kLoadsQ>{}, [&](int l) { load_q(k0, prev_stage, l); });
       } else {
-        step(fa0, fb0, fa1, fb1, stage, kk + 1, std::integral_constant<int, 0>{}, [](int) {});
+        first_half(fb0, stage, kk, Zero{}, [](int) {});
       }
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      second_half(fb0, fb1, stage, kk + 1, Zero{}, [](int) {});
+      __builtin_amdgcn_s_waitcnt(kWaitLds);
+      __builtin_amdgcn_sched_barrier(0);
+      first_half(fb1, stage, kk + 1, Zero{}, [](int) {});
       if (kk + 2 < kSteps) {
         __builtin_amdgcn_s_waitcnt(kWaitLds);
         __builtin_amdgcn_sched_barrier(0);
-        step(fa1, fb1, fa0, fb0, stage, kk + 2, std::integral_constant<int, 0>{}, [](int) {});
+        second_half(fb1, fb0, stage, kk + 2, Zero{}, [](int) {});
       } else {
-        // last step of the slab: the slab after it must have landed (the STAGES - 2 younger ones may be in flight);
-        // behind the barrier this slab's stage is free and its refill starts with the P rows
+        // last half step of the slab: the slab after it must have landed (the STAGES - 2 younger ones may be in
+        // flight); behind the barrier this slab's stage is free and its refill starts with the P rows
         __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         const int k0 = k0_clamped(it + STAGES);
-        step(fa1, fb1, fa0, fb0, next_stage, 0, std::integral_constant<int, kLoadsP>{}, [&](int l) { load_p(k0, stage, l); });
+        second_half(fb1, fb0, next_stage, 0, std::integral_constant<int, kLoadsP>{}, [&](int l) { load_p(k0, stage, l); });
       }
     }
     stage = next_stage;
@@ -295,27 +316,24 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   __builtin_amdgcn_s_waitcnt(0x0070);  // the loads past the end of the walk have landed too; LDS is free
 
   // ---- K pieces: park the fp32 partial tile (row-major BM x BN); the fix-up kernel sums the pieces and
-  // runs the epilogue.  Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
+  // runs the epilogue.  Accumulator register r of lane l holds C[4*(l/16) + r][l%16] of its 16x16 tile.
+  const int lcol = wave_n * kWaveN + (lane & 15);
+  const int lrow = wave_m * kWaveM + (lane >> 4) * 4;
   if (!whole) {
     float* mine = sched.partials + (static_cast<int64_t>(piece_tile) * sched.splits + split) * (BM * BN);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = wave_n * kWaveN + j * 32 + (lane & 31);
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = wave_m * kWaveM + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-          mine[row * BN + col] = acc[i][j][r];
-        }
-      }
+        for (int r = 0; r < 4; ++r) mine[(lrow + i * 16 + r) * BN + lcol + j * 16] = acc[i][j][r];
     return;
   }
 
 
   // ---- epilogue, staged through LDS so that HBM only sees whole 16-byte-per-lane, row-contiguous accesses.
-  // Accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile: written
-  // straight from registers that would be 2-byte stores for C and 8-byte stores scattered over 32 rows for
+  // Accumulator register r of lane l holds C[4*(l/16) + r][l%16] of its 16x16 tile: written
+  // straight from registers that would be 2-byte stores for C and 8-byte stores scattered over 16 rows for
   // the transpose.  Instead: D tile -> LDS (coalesced), combine, C tile -> LDS -> HBM, transposed tile -> LDS -> HBM.
   const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
@@ -346,16 +364,14 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
     __syncthreads();
   }
-  const int lcol = wave_n * kWaveN + (lane & 31);
-  const int lrow = wave_m * kWaveM + frag_half * 4;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < 4; ++r) {
         float v = a.alpha * acc[i][j][r];
-        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * BN + lcol + j * 32]);
+        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 16 + r) * BN + lcol + j * 16]);
         acc[i][j][r] = v;
       }
   if (D != nullptr) __syncthreads();  // the D tile has been consumed
@@ -365,9 +381,8 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          stage_c[(lrow + i * 32 + (r >> 2) * 8 + (r & 3)) * kLdS + lcol + j * 32] =
-              __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
+        for (int r = 0; r < 4; ++r)
+          stage_c[(lrow + i * 16 + r) * kLdS + lcol + j * 16] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
     __syncthreads();
     for (int c = tid; c < BM * kRowChunks; c += kThreads) {
       const int r = c / kRowChunks, cc = c - r * kRowChunks;
@@ -382,11 +397,11 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        u32x2 four = {pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]), pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3])};
-        *reinterpret_cast<u32x2*>(stage_c + (lcol + j * 32) * kLdT + lrow + i * 32 + q * 8) = four;
-      }
+    {
+      // the four registers of a tile are four consecutive rows of one column: four consecutive elements of a transposed row
+      u32x2 four = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
+      *reinterpret_cast<u32x2*>(stage_c + (lcol + j * 16) * kLdT + lrow + i * 16) = four;
+    }
   __syncthreads();
   for (int c = tid; c < BN * kColChunks; c += kThreads) {
     const int r = c / kColChunks, cc = c - r * kColChunks;
