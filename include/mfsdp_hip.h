@@ -89,9 +89,9 @@ int mfsdp_copy_rank_segments_to_full(const void* local, int64_t local_numel, voi
  *
  * workspace == NULL: one tile slot per (segment, tile index up to max_numel), the reference's launch shape; needs
  * nothing besides the arguments and is safe on concurrent streams.  workspace != NULL (8-byte aligned, at least
- * mfsdp_copy_rank_segments_workspace_bytes(n_segments) bytes, not shared by calls that may overlap): a scan kernel
- * writes the segments' running tile counts there and a persistent grid cuts the copy by bytes instead of by
- * segment -- the shape to use when segment lengths differ widely.
+ * mfsdp_copy_rank_segments_workspace_bytes(n_segments) bytes, not shared by calls that may overlap): two small
+ * kernels write the segments' running tile counts there (per block of 1024 segments, plus one offset per block) and
+ * the copy grid is cut by bytes instead of by segment -- the shape to use when segment lengths differ widely.
  */
 int64_t mfsdp_copy_rank_segments_workspace_bytes(int64_t n_segments);
 int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_numel, void* output, int64_t output_numel,
@@ -102,7 +102,7 @@ int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_num
 /*
  * The device-metadata copy above in its byte-balanced launch shape, for callers that cannot allocate: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The
- * segments' running tile counts go into a 1 MiB array that is part of the library's device image (every GPU the
+ * segments' running tile counts go into an array of 1 MiB + 2 KiB that is part of the library's device image (every GPU the
  * library runs on holds its own copy until the process ends) instead of a caller's workspace, so the call neither
  * allocates nor frees anything; more than MFSDP_NOALLOC_MAX_SEGMENTS segments are rejected with
  * MFSDP_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two

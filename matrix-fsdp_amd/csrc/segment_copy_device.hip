@@ -15,10 +15,10 @@
 // Two launch shapes:
 //   * uniform: one tile slot per (segment, tile index up to the longest segment), as the reference's
 //     (tiles, segments) grid; needs no memory besides the arguments, slots past a segment's end exit at once;
-//   * balanced: a one-workgroup scan writes the running tile count of the segments into a caller-provided (or the
-//     library's static) scratch array, and a persistent grid takes chunks of consecutive tiles, finds the chunk's
-//     first segment by bisection and walks on from there -- the work is cut by bytes, so one very long segment
-//     beside many short ones costs no empty slots.
+//   * balanced: two small kernels write the running tile counts of the segments (per block of 1024 segments, plus one
+//     offset per block) into a caller-provided (or the library's static) scratch array, and the waves of the copy
+//     grid take one tile each (striding on when the grid is capped) and find its segment by bisection -- the work
+//     is cut by bytes, so one very long segment beside many short ones costs no empty slots.
 #include "mfsdp_common.h"
 
 #include <algorithm>
@@ -32,15 +32,25 @@ constexpr int kUnroll = 4;
 constexpr int kTileVectors = kWave * kUnroll;
 constexpr int kCopyThreads = 256;
 constexpr int kWavesPerBlock = kCopyThreads / kWave;
-constexpr int kScanThreads = 1024;
-constexpr int kScanPerThread = 8;
-constexpr int kChunkTiles = 8;  // consecutive tiles one bisection serves (32 KiB at V = 16)
+constexpr int kCountThreads = 256;
+constexpr int kCountPerThread = 4;
+constexpr int kBlockSegments = kCountThreads * kCountPerThread;  // segments whose tile counts one workgroup sums
+constexpr int kBlockShift = 10;
+static_assert(kBlockSegments == 1 << kBlockShift, "block of segments");
+// Consecutive tiles one bisection serves, and the workgroups per CU the balanced grid is capped at.  Measured on the
+// 21 250 row segments of a hidden4096 rank shard: (8 tiles, 4 per CU) 50 us, (4, 16) 48 us, (1, 64) 45 us, (1, 256) 59 us;
+// eight segments of 50 MB: 163, 176, 148, 155 us.  Many short-lived waves beat few long-lived ones, as in the other
+// copy kernels, until the empty workgroups of the upper-bound grid cost more than they hide.
+constexpr int kChunkTiles = 1;
+constexpr int kBalancedBlocksPerCu = 64;
 constexpr int kMaxDevices = 64;
 
-// Scratch of the entry point that allocates nothing: the running tile counts of up to kStaticMaxSegments segments.
-constexpr int64_t kStaticScratchBytes = 1 << 20;
-constexpr int64_t kStaticMaxSegments = kStaticScratchBytes / 8 - 1;
-static_assert(kStaticMaxSegments == MFSDP_NOALLOC_MAX_SEGMENTS, "the header states the limit");
+// Scratch of the entry point that allocates nothing: the tile-count tables of up to kStaticMaxSegments segments.
+constexpr int64_t kStaticScratchBytes = (1 << 20) + 2048;
+constexpr int64_t kStaticMaxSegments = MFSDP_NOALLOC_MAX_SEGMENTS;
+// entries of 8 bytes the tile-count tables of n segments take: n + 1 running counts, one offset per block of segments + 1
+constexpr int64_t table_entries(int64_t n) { return n + 1 + (n + kBlockSegments - 1) / kBlockSegments + 1; }
+static_assert(table_entries(kStaticMaxSegments) * 8 <= kStaticScratchBytes, "the header states the limit");
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -69,21 +79,44 @@ struct Geometry {
   uint64_t tiles;
 };
 
+// What the addresses of a segment allow, from the low 32 bits of its first source and destination byte (V <= 16, so
+// the low four bits decide): V and the destination's offset inside its V-byte vector.
+__device__ __forceinline__ void vector_shape(uint32_t src_lo, uint32_t dst_lo, uint32_t* vec, uint32_t* lead) {
+  const uint32_t d = (src_lo - dst_lo) & 15u;
+  *vec = d ? (d & (0u - d)) : 16u;  // lowest set bit of the difference, 16 when the two are congruent mod 16
+  *lead = dst_lo & (*vec - 1);
+}
+
+// True when the segment is copied at all: not empty, and inside both tensors.
+__device__ __forceinline__ bool segment_is_live(const SegmentCopyArgs& a, int64_t gs, int64_t ls, int64_t n) {
+  return n > 0 && gs >= 0 && ls >= 0 && ls <= a.local_numel - n && gs <= a.output_numel - n;
+}
+
+// Tiles of a segment from its three metadata values (zero when it is not copied): the part of the geometry the scan
+// needs, in 32-bit arithmetic wherever the low bits decide.
+__device__ __forceinline__ uint64_t segment_tiles(const SegmentCopyArgs& a, int64_t gs, int64_t ls, int64_t n) {
+  if (!segment_is_live(a, gs, ls, n)) return 0;
+  n = n < a.limit ? n : a.limit;
+  const uint32_t eb = static_cast<uint32_t>(a.elem_bytes);
+  uint32_t vec, lead;
+  vector_shape(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(a.local)) + static_cast<uint32_t>(ls) * eb,
+               static_cast<uint32_t>(reinterpret_cast<uintptr_t>(a.output)) + static_cast<uint32_t>(gs) * eb, &vec, &lead);
+  const uint64_t n_vec = (static_cast<uint64_t>(n) * eb + lead + vec - 1) >> __builtin_ctz(vec);
+  return (n_vec + kTileVectors - 1) / kTileVectors;
+}
+
 // Geometry of segment s; a segment that is empty or leaves either tensor gets zero tiles (it is not copied).
 __device__ __forceinline__ Geometry segment_geometry(const SegmentCopyArgs& a, int64_t s) {
   Geometry g{};
   const int64_t gs = a.global_starts[s], ls = a.local_starts[s];
   int64_t n = a.numels[s];
-  if (n <= 0 || gs < 0 || ls < 0 || ls > a.local_numel - n || gs > a.output_numel - n) return g;
+  if (!segment_is_live(a, gs, ls, n)) return g;
   n = n < a.limit ? n : a.limit;
   g.src = a.local + ls * a.elem_bytes;
   g.dst = a.output + gs * a.elem_bytes;
   g.nbytes = n * a.elem_bytes;
-  const uint64_t diff = reinterpret_cast<uint64_t>(g.src) - reinterpret_cast<uint64_t>(g.dst);
-  const uint64_t low = diff & (~diff + 1);  // lowest set bit, 0 when the addresses are congruent to every power of two
-  g.vec = (low == 0 || low >= 16) ? 16u : static_cast<uint32_t>(low);
-  g.lead = static_cast<uint32_t>(reinterpret_cast<uint64_t>(g.dst) & (g.vec - 1));
-  g.n_vec = (static_cast<uint64_t>(g.nbytes) + g.lead + g.vec - 1) / g.vec;
+  vector_shape(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(g.src)), static_cast<uint32_t>(reinterpret_cast<uintptr_t>(g.dst)), &g.vec, &g.lead);
+  g.n_vec = (static_cast<uint64_t>(g.nbytes) + g.lead + g.vec - 1) >> __builtin_ctz(g.vec);  // V is a power of two
   g.tiles = (g.n_vec + kTileVectors - 1) / kTileVectors;
   return g;
 }
@@ -183,67 +216,92 @@ segment_copy_uniform_kernel(SegmentCopyArgs a, uint64_t slots_per_segment, uint6
   }
 }
 
-// ---- balanced launch shape, step 1: prefix[0] = 0, prefix[s + 1] = tiles of segments 0..s.  One workgroup.
-__global__ void __launch_bounds__(kScanThreads)
-segment_tile_scan_kernel(SegmentCopyArgs a, uint64_t* __restrict__ prefix) {
-  __shared__ uint64_t wave_sums[kScanThreads / kWave];
-  __shared__ uint64_t block_total;
+// ---- balanced launch shape, step 1.  The running tile counts are kept in two levels, so that many workgroups can
+// build them: counts[s + 1] = tiles of the segments from the start of s's block of 1024 up to and including s, and
+// block_offsets[b] = tiles of all blocks before b (block_offsets[n_blocks] = all tiles).  running_count() below puts
+// the two together: tiles of the segments before s.
+__global__ void __launch_bounds__(kCountThreads)
+segment_tile_count_kernel(SegmentCopyArgs a, uint64_t* __restrict__ counts, uint64_t* __restrict__ block_offsets) {
+  __shared__ uint64_t wave_sums[kCountThreads / kWave];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  uint64_t carry = 0;
-  if (tid == 0) prefix[0] = 0;
-  for (int64_t base = 0; base < a.n_segments; base += static_cast<int64_t>(kScanThreads) * kScanPerThread) {
-    const int64_t first = base + static_cast<int64_t>(tid) * kScanPerThread;
-    uint64_t mine[kScanPerThread];
-    uint64_t sum = 0;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kBlockSegments + static_cast<int64_t>(tid) * kCountPerThread;
+  if (blockIdx.x == 0 && tid == 0) {
+    counts[0] = 0;
+    block_offsets[0] = 0;
+  }
+  uint64_t mine[kCountPerThread];
+  uint64_t sum = 0;
 #pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) {
-      mine[i] = first + i < a.n_segments ? segment_geometry(a, first + i).tiles : 0;
-      sum += mine[i];
-    }
-    // inclusive scan of the per-thread sums: within the wave by shuffles, across the 16 waves through LDS
-    uint64_t incl = sum;
+  for (int i = 0; i < kCountPerThread; ++i) {
+    const int64_t at = first + i < a.n_segments ? first + i : a.n_segments - 1;
+    mine[i] = first + i < a.n_segments ? segment_tiles(a, a.global_starts[at], a.local_starts[at], a.numels[at]) : 0;
+    sum += mine[i];
+  }
+  // inclusive scan of the per-thread sums: within the wave by shuffles, across the waves through LDS
+  uint64_t incl = sum;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint64_t up = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += up;
+  }
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  uint64_t before = 0;
+  for (int w = 0; w < wave; ++w) before += wave_sums[w];
+  uint64_t running = before + incl - sum;  // tiles of the block's segments before this thread's first
+#pragma unroll
+  for (int i = 0; i < kCountPerThread; ++i) {
+    running += mine[i];
+    if (first + i < a.n_segments) counts[first + i + 1] = running;
+  }
+  if (tid == kCountThreads - 1) block_offsets[blockIdx.x + 1] = before + incl;  // the block's total, summed up by the next kernel
+}
+
+// One wavefront turns the block totals (entries 1 .. n_blocks) into running sums, 64 at a time.
+__global__ void __launch_bounds__(kWave)
+block_offset_kernel(uint64_t* __restrict__ block_offsets, int64_t n_blocks) {
+  const int lane = threadIdx.x;
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < n_blocks; base += kWave) {
+    const int64_t at = base + lane;
+    uint64_t incl = at < n_blocks ? block_offsets[at + 1] : 0;
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
       const uint64_t up = __shfl_up(incl, d, kWave);
       if (lane >= d) incl += up;
     }
-    if (lane == kWave - 1) wave_sums[wave] = incl;
-    __syncthreads();
-    uint64_t before = carry;
-    for (int w = 0; w < wave; ++w) before += wave_sums[w];
-    if (tid == kScanThreads - 1) block_total = before + incl - carry;
-    uint64_t running = before + incl - sum;  // tiles of every segment before this thread's first
-#pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) {
-      running += mine[i];
-      if (first + i < a.n_segments) prefix[first + i + 1] = running;
-    }
-    __syncthreads();
-    carry += block_total;
-    __syncthreads();  // wave_sums / block_total are rewritten by the next round
+    if (at < n_blocks) block_offsets[at + 1] = carry + incl;
+    carry += __shfl(incl, kWave - 1, kWave);
   }
 }
 
-// ---- balanced launch shape, step 2: persistent waves take chunks of consecutive tiles.
+// Tiles of the segments before s, 0 <= s <= n_segments.
+__device__ __forceinline__ uint64_t running_count(const uint64_t* __restrict__ counts, const uint64_t* __restrict__ block_offsets, int64_t s) {
+  return s == 0 ? 0 : counts[s] + block_offsets[(s - 1) >> kBlockShift];
+}
+
+// ---- balanced launch shape, step 2: every wave takes chunks of chunk_tiles consecutive tiles, chunk = wave, wave + waves, ...
 __global__ void __launch_bounds__(kCopyThreads)
-segment_copy_balanced_kernel(SegmentCopyArgs a, const uint64_t* __restrict__ prefix, uint32_t chunk_tiles) {
+segment_copy_balanced_kernel(SegmentCopyArgs a, const uint64_t* __restrict__ counts, const uint64_t* __restrict__ block_offsets,
+                             uint32_t chunk_tiles) {
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * kWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWavesPerBlock;
-  const uint64_t total = prefix[a.n_segments];
+  auto prefix = [&](int64_t at) { return running_count(counts, block_offsets, at); };
+  const uint64_t total = prefix(a.n_segments);
   const uint64_t n_chunks = (total + chunk_tiles - 1) / chunk_tiles;
   for (uint64_t chunk = wave; chunk < n_chunks; chunk += n_waves) {
     uint64_t t = chunk * chunk_tiles;
     const uint64_t t_end = t + chunk_tiles < total ? t + chunk_tiles : total;
-    // the segment holding tile t: prefix[s] <= t < prefix[s + 1]  (prefix[0] = 0 <= t < total = prefix[n_segments])
+    // the segment holding tile t: prefix(s) <= t < prefix(s + 1)  (prefix(0) = 0 <= t < total = prefix(n_segments))
     int64_t lo = 0, hi = a.n_segments;
     while (hi - lo > 1) {
       const int64_t mid = lo + ((hi - lo) >> 1);
-      if (prefix[mid] <= t) lo = mid; else hi = mid;
+      if (prefix(mid) <= t) lo = mid; else hi = mid;
     }
     int64_t s = lo;
     while (t < t_end && s < a.n_segments) {
-      const uint64_t seg_begin = prefix[s], seg_end = prefix[s + 1];
+      const uint64_t seg_begin = prefix(s), seg_end = prefix(s + 1);
       if (t >= seg_end) { ++s; continue; }
       const Geometry g = segment_geometry(a, s);
       const uint64_t upto = t_end < seg_end ? t_end : seg_end;
@@ -294,14 +352,21 @@ uint64_t max_tiles_per_segment(const SegmentCopyArgs& a) {
   return (vectors + kTileVectors - 1) / kTileVectors;
 }
 
-int launch_balanced(const SegmentCopyArgs& a, uint64_t* prefix, hipStream_t stream) {
-  hipLaunchKernelGGL(segment_tile_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, a, prefix);
-  MFSDP_CHECK_LAUNCH("segment_tile_scan_kernel");
+int launch_balanced(const SegmentCopyArgs& a, uint64_t* tables, hipStream_t stream) {
+  uint64_t* counts = tables;                          // n_segments + 1 entries
+  uint64_t* block_offsets = tables + a.n_segments + 1;  // n_blocks + 1 entries
+  const int64_t n_blocks = (a.n_segments + kBlockSegments - 1) / kBlockSegments;
+  if (n_blocks > (int64_t{1} << 31) - 1) return fail(MFSDP_ERR_UNSUPPORTED, "%lld segments are beyond the grid", static_cast<long long>(a.n_segments));
+  hipLaunchKernelGGL(segment_tile_count_kernel, dim3(static_cast<uint32_t>(n_blocks)), dim3(kCountThreads), 0, stream, a, counts, block_offsets);
+  MFSDP_CHECK_LAUNCH("segment_tile_count_kernel");
+  hipLaunchKernelGGL(block_offset_kernel, dim3(1), dim3(kWave), 0, stream, block_offsets, n_blocks);
+  MFSDP_CHECK_LAUNCH("block_offset_kernel");
   const uint64_t bound = static_cast<uint64_t>(a.n_segments) * max_tiles_per_segment(a);
+  // one tile per wave while the grid can hold them all (excess waves leave at once; beyond that the waves stride on)
   const uint64_t want = (bound + kChunkTiles * kWavesPerBlock - 1) / (kChunkTiles * kWavesPerBlock);
-  const uint64_t cap = static_cast<uint64_t>(device_cu_count()) * 4;
+  const uint64_t cap = static_cast<uint64_t>(device_cu_count()) * kBalancedBlocksPerCu;
   const dim3 grid(static_cast<uint32_t>(std::max<uint64_t>(1, std::min(want, cap))));
-  hipLaunchKernelGGL(segment_copy_balanced_kernel, grid, dim3(kCopyThreads), 0, stream, a, prefix, static_cast<uint32_t>(kChunkTiles));
+  hipLaunchKernelGGL(segment_copy_balanced_kernel, grid, dim3(kCopyThreads), 0, stream, a, counts, block_offsets, static_cast<uint32_t>(kChunkTiles));
   MFSDP_CHECK_LAUNCH("segment_copy_balanced_kernel");
   return MFSDP_OK;
 }
@@ -330,7 +395,7 @@ int static_scratch(uint64_t** out) {
 using namespace mfsdp;
 
 extern "C" int64_t mfsdp_copy_rank_segments_workspace_bytes(int64_t n_segments) {
-  return n_segments < 0 ? 0 : (n_segments + 1) * 8;
+  return n_segments < 0 ? 0 : table_entries(n_segments) * 8;
 }
 
 extern "C" int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_numel, void* output, int64_t output_numel,

@@ -85,6 +85,23 @@ def test_one_long_segment_beside_many_short_ones(balanced):
     assert_same_bits(out, want)
 
 
+@pytest.mark.parametrize("n_seg", [1023, 1024, 1025, 2048, 3333])
+def test_segment_counts_around_the_blocks_of_the_tile_count_tables(n_seg):
+    """The balanced shape keeps its running tile counts per block of 1024 segments plus one offset per block: segment
+    counts just below, at and above the block size, with empty segments and one long segment in the last block."""
+    rng = np.random.default_rng(n_seg)
+    lengths = [int(rng.integers(0, 700)) if rng.integers(0, 5) else 0 for _ in range(n_seg)]
+    lengths[-1] = 40_000
+    lengths[n_seg // 2] = 0
+    gs, ls, ln, local_n, out_n = random_segments(rng, n_seg, 0, lengths=lengths)
+    host_local, host_out = random_values(local_n, torch.bfloat16, 5), random_values(out_n, torch.bfloat16, 6)
+    want = host_out.clone()
+    CO.copy_rank_segments_to_full_kernel(host_local, want, gs, ls, ln, max(ln))
+    out = host_out.to(DEV)
+    run_device(host_local.to(DEV), out, gs, ls, ln, max(ln), True)
+    assert_same_bits(out, want)
+
+
 @pytest.mark.parametrize("balanced", [False, True], ids=["uniform", "balanced"])
 def test_max_numel_smaller_than_a_segment_truncates_like_the_reference_grid(balanced):
     gs, ls, ln = [0, 2000, 2600], [0, 1500, 1100], [1500, 300, 400]
