@@ -10,17 +10,19 @@ namespace mfsdp {
 // C = bf16( alpha * (P * Q^T) + beta * D ), fp32 accumulation.
 //   P: M x K row-major (ldp), Q: N x K row-major (ldq), D / C: M x N row-major (ldd / ldc).
 //   M, N multiples of 256 and K a multiple of 64 (callers zero-pad their operands).
-//   D may be null (beta ignored).  CT, when non-null, also receives the transpose: CT[n][m] = C[m][n]
+//   D may be null (beta ignored); with D its transpose DT is passed too.  CT, when non-null, also receives the transpose: CT[n][m] = C[m][n]
 //   (ldct); with skip_c only CT is written.  symmetric: P*Q^T is known to be symmetric (M == N); only tiles on or below the diagonal are
 //   computed and each off-diagonal tile is also written mirrored into C.
 struct GemmNtArgs {
   const void* P;
   const void* Q;
   const void* D;
+  const void* DT;  // D transposed (N x M row-major, lddt; D itself when D is symmetric), required with D: tiles computed
+                   // whole start their accumulators from it (the K-split pieces' fix-up reads D)
   void* C;
   void* CT;
   int M, N, K;
-  int ldp, ldq, ldd, ldc, ldct;
+  int ldp, ldq, ldd, ldc, ldct, lddt;
   float alpha, beta;
   int symmetric;
   int skip_c;  // general product with CT set: write only the transposed output

@@ -169,13 +169,49 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int i = 0; i < kLoadsQ; ++i) load_q(k0, stage, i);
   };
 
+  // Accumulator register r of lane l holds C[4*(l/16) + r][l%16] of its 16x16 tile.
+  const int lcol = wave_n * kWaveN + (lane & 15);
+  const int lrow = wave_m * kWaveM + (lane >> 4) * 4;
+  // A whole tile whose D operand is also at hand transposed starts from it instead of adding it at the end:
+  // acc = (beta / alpha) D, so that alpha * acc is alpha P Q^T + beta D with one rounding, as before.  The four
+  // registers of an MFMA tile are four consecutive rows of one column, i.e. four consecutive elements (8 bytes) of a
+  // row of D^T, which come straight from global memory in the accumulator's layout and go out with the first slabs.
+  // (A D tile fetched behind the main loop has to be staged through LDS, since its rows do not match the accumulator
+  // layout, and picked up with 2-byte LDS reads: 5 of the 121 microseconds of a 256x256 tile with K = 4096.  The
+  // fetch itself stays what it is wherever it sits: every CU wants its 128 KiB at the same moment.)
+  const bool start_from_d = whole && a.DT != nullptr;
   f32x4 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
+  u32x2 d_raw[TM][TN];
+  if (start_from_d) {
+    const uint16_t* __restrict__ DT = static_cast<const uint16_t*>(a.DT);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+      for (int i = 0; i < TM; ++i)  // consecutive i: consecutive 32-byte pieces of the same rows of D^T
+        d_raw[i][j] = *reinterpret_cast<const u32x2*>(DT + static_cast<int64_t>(col0 + lcol + j * 16) * a.lddt + row0 + lrow + i * 16);
+  }
+  // (the values are turned into accumulators behind the first slab loads, so that the two fetches overlap)
+  auto start_accumulators = [&]() {
+    if (start_from_d) {
+      const float scale = a.beta / a.alpha;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j][0] = scale * __uint_as_float(d_raw[i][j].x << 16);
+          acc[i][j][1] = scale * __uint_as_float(d_raw[i][j].x & 0xffff0000u);
+          acc[i][j][2] = scale * __uint_as_float(d_raw[i][j].y << 16);
+          acc[i][j][3] = scale * __uint_as_float(d_raw[i][j].y & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+    }
+  };
 
   // 16x16x32 MFMA operands: lane l supplies row l % 16 of its 16-row block and the 8 k values of chunk l / 16 of
   // the 32 wide step.  (At equal peak rate this shape draws less power than 32x32x16 on operands with random
@@ -215,6 +251,8 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       stream_p(k0_clamped(sidx), sidx);
       if (sidx + 1 < STAGES) stream_q(k0_clamped(sidx), sidx);  // the Q rows of the last one go out under the first MFMAs
     }
+    __builtin_amdgcn_sched_barrier(0);  // the slab loads are on their way before the D values are waited for
+    start_accumulators();
     constexpr int kAfterFirst = (STAGES - 2) * kLoadsPerSlab + kLoadsP;
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kAfterFirst & 0xF) | ((kAfterFirst >> 4) << 14));
     __syncthreads();
@@ -223,6 +261,8 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int i = 0; i < TMH; ++i) fa_lo[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 16 * BK);
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb0[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 16 * BK);
+  } else {
+    start_accumulators();
   }
   // One half step: the TMH x TN MFMAs on the fragments in hand (use_a for tile rows row0.., use_b), kReads LDS
   // reads (read(r), one behind each of the first MFMAs) and kLoads slab loads, interleaved instruction by
@@ -316,9 +356,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   __builtin_amdgcn_s_waitcnt(0x0070);  // the loads past the end of the walk have landed too; LDS is free
 
   // ---- K pieces: park the fp32 partial tile (row-major BM x BN); the fix-up kernel sums the pieces and
-  // runs the epilogue.  Accumulator register r of lane l holds C[4*(l/16) + r][l%16] of its 16x16 tile.
-  const int lcol = wave_n * kWaveN + (lane & 15);
-  const int lrow = wave_m * kWaveM + (lane >> 4) * 4;
+  // runs the epilogue.
   if (!whole) {
     float* mine = sched.partials + (static_cast<int64_t>(piece_tile) * sched.splits + split) * (BM * BN);
 #pragma unroll
@@ -334,8 +372,8 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // ---- epilogue, staged through LDS so that HBM only sees whole 16-byte-per-lane, row-contiguous accesses.
   // Accumulator register r of lane l holds C[4*(l/16) + r][l%16] of its 16x16 tile: written
   // straight from registers that would be 2-byte stores for C and 8-byte stores scattered over 16 rows for
-  // the transpose.  Instead: D tile -> LDS (coalesced), combine, C tile -> LDS -> HBM, transposed tile -> LDS -> HBM.
-  const uint16_t* __restrict__ D = static_cast<const uint16_t*>(a.D);
+  // the transpose.  Instead: C tile -> LDS -> HBM, transposed tile -> LDS -> HBM.  (The D operand is already in the
+  // accumulators.)
   uint16_t* __restrict__ C = static_cast<uint16_t*>(a.C);
   uint16_t* __restrict__ CT = static_cast<uint16_t*>(a.CT);
   int ldct = a.ldct;
@@ -348,33 +386,12 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   constexpr int kLdT = BM + 8;  // row pitch of the staged transposed tile
   constexpr int kRowChunks = BN / 8, kColChunks = BM / 8;
   __syncthreads();  // every wave is done reading the slab stages
-  if (D != nullptr) {
-    // the D tile streams into LDS (unpadded BM x BN) with all of its loads in flight at once; fetched through
-    // registers, the loads of a thread run one after the other and their latencies add up
-    constexpr int kRowsPerDLoad = 512 / BN;  // D rows one wave-level 1 KiB load covers
-    constexpr int kDLoads = BM / kRowsPerDLoad / kWaves;
-    static_assert(512 % BN == 0 && BM % (kRowsPerDLoad * kWaves) == 0 && kDLoads < 64, "D tile must divide over the waves");
-    const int d_row = lane / kRowChunks, d_chunk = lane % kRowChunks;
-#pragma unroll
-    for (int i = 0; i < kDLoads; ++i) {
-      const int r0 = (i * kWaves + wave) * kRowsPerDLoad;
-      const uint16_t* src = D + static_cast<int64_t>(row0 + r0 + d_row) * a.ldd + col0 + d_chunk * 8;
-      __builtin_amdgcn_global_load_lds(src, stage_c + r0 * BN, 16, 0, 0);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
-    __syncthreads();
-  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = a.alpha * acc[i][j][r];
-        if (D != nullptr) v += a.beta * bf16_bits_to_float(stage_c[(lrow + i * 16 + r) * BN + lcol + j * 16]);
-        acc[i][j][r] = v;
-      }
-  if (D != nullptr) __syncthreads();  // the D tile has been consumed
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = a.alpha * acc[i][j][r];
   if (!a.skip_c) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -603,6 +620,9 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
       (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
+  if ((a.D != nullptr) != (a.DT != nullptr)) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: D and its transpose come together");
+  if (a.DT && (a.lddt < a.M || (a.lddt % 4) || reinterpret_cast<uintptr_t>(a.DT) % 8 || a.alpha == 0.0f))
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: the transposed D needs alpha != 0, 8-byte alignment and a leading dimension >= M that is a multiple of 4");
   const GemmTuning tuning = tuning_snapshot();
   // Slabs of 32 (three to five deep) were measured too: each slab row is then half a 128-byte line, the vector
   // cache looks every line up twice, and the products run 15-25 % slower than with slabs of 64 two deep.
