@@ -83,14 +83,14 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.A; g.Q = w.A; g.D = w.A; g.C = w.B; g.CT = nullptr;
-    g.DT = w.A; g.lddt = w.mp;  // A is symmetric
+    g.d_transposed_is_q = 1;  // A is symmetric
     g.M = w.mp; g.N = w.mp; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.mp; g.ldc = w.mp; g.ldct = 0;
     g.alpha = c; g.beta = b; g.symmetric = 1; g.shared = shared;
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
     g = GemmNtArgs{};
     g.P = w.B; g.Q = w.XT[cur]; g.D = w.X[cur]; g.C = w.X[nxt]; g.CT = w.XT[nxt];
-    g.DT = w.XT[cur]; g.lddt = w.mp;
+    g.d_transposed_is_q = 1;  // Q = X^T
     g.M = w.mp; g.N = w.np; g.K = w.mp;
     g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.np; g.ldc = w.np; g.ldct = w.mp;
     g.alpha = 1.0f; g.beta = a; g.symmetric = 0;

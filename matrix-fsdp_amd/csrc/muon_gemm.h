@@ -10,22 +10,23 @@ namespace mfsdp {
 // C = bf16( alpha * (P * Q^T) + beta * D ), fp32 accumulation.
 //   P: M x K row-major (ldp), Q: N x K row-major (ldq), D / C: M x N row-major (ldd / ldc).
 //   M, N multiples of 256 and K a multiple of 64 (callers zero-pad their operands).
-//   D may be null (beta ignored); with D its transpose DT is passed too.  CT, when non-null, also receives the transpose: CT[n][m] = C[m][n]
+//   D may be null (beta ignored); with D, Q must hold its transpose (d_transposed_is_q, K >= M).  CT, when non-null, also receives the transpose: CT[n][m] = C[m][n]
 //   (ldct); with skip_c only CT is written.  symmetric: P*Q^T is known to be symmetric (M == N); only tiles on or below the diagonal are
 //   computed and each off-diagonal tile is also written mirrored into C.
 struct GemmNtArgs {
   const void* P;
   const void* Q;
   const void* D;
-  const void* DT;  // D transposed (N x M row-major, lddt; D itself when D is symmetric), required with D: tiles computed
-                   // whole start their accumulators from it (the K-split pieces' fix-up reads D)
   void* C;
   void* CT;
   int M, N, K;
-  int ldp, ldq, ldd, ldc, ldct, lddt;
+  int ldp, ldq, ldd, ldc, ldct;
   float alpha, beta;
   int symmetric;
   int skip_c;  // general product with CT set: write only the transposed output
+  int d_transposed_is_q;  // the caller's word that Q holds D^T (Q[n][k] == D[k][n] for k < M): required with D, whose
+                          // values whole tiles pick out of the Q slabs on their way through LDS (the fix-up of K-split
+                          // pieces reads D itself)
   int shared;  // other matrices' products run beside this one on other streams: a symmetric product then takes the
                // 256 x 256 tiles even where their triangle fills only part of the CUs (the rest works for the others)
 };

@@ -3,11 +3,11 @@
 // Both operands are K-contiguous (an "NT" product), which is what every Newton-Schulz product
 // reduces to once X and X^T are both kept: X X^T, A A^T (A symmetric) and B (X^T)^T.  A workgroup owns
 // a BM x BN tile of C; its waves each own a (BM/WM) x (BN/WN) sub-tile built from 16x16x32 bf16 MFMAs
-// with fp32 accumulators.  K is walked in slabs of BK (64 or 32): the slab of P and Q is staged in LDS as
+// with fp32 accumulators.  K is walked in slabs of BK = 64: the slab of P and Q is staged in LDS as
 // rows of BK bf16 whose 16-byte chunks are XOR-swizzled with the row index: the LDS has 64 banks of 4
 // bytes, 256 / (2 BK) rows span them once, so any 16 consecutive rows read at one logical chunk touch every
 // bank exactly once and the 128-bit fragment reads are bank-conflict free.  STAGES slabs are resident: the
-// next ones stream from HBM straight into LDS (global_load ... lds, no register round trip) while the
+// next ones stream from HBM straight into LDS (buffer_load ... lds, no register round trip) while the
 // current one feeds the MFMAs.
 //
 // Tile scheduling.  Tiles are handed to workgroups so that the groups sharing an XCD (block ids
@@ -23,6 +23,7 @@
 #include <algorithm>
 #include <mutex>
 #include <type_traits>
+#include <utility>
 
 namespace mfsdp {
 namespace {
@@ -124,7 +125,7 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // dimensions every row of a slab maps to the same memory channel, and tiles marching in lock step would all
   // queue on that one channel.
   const int n_slabs = ks_end - ks_begin;
-  const int k_start = (sched.stagger > 0 && n_slabs > 0) ? static_cast<int>((static_cast<int64_t>(logical) * sched.stagger) % n_slabs) : 0;
+  const int k_start = (sched.stagger > 0 && n_slabs > 0 && !(whole && a.D != nullptr)) ? static_cast<int>((static_cast<int64_t>(logical) * sched.stagger) % n_slabs) : 0;
   auto k0_of = [&](int i) {
     int slab = i + k_start;
     if (slab >= n_slabs) slab -= n_slabs;
@@ -144,21 +145,33 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // position c ^ ((r / kRowsPerSweep) % kChunks).  One wave-level direct-to-LDS load fills 1 KiB = kRowsPerLoad
   // rows: lane l lands at row l / kChunks, position l % kChunks, and therefore fetches the global chunk the
   // swizzle maps there.  Wave w takes the row groups w, w + kWaves, ...
-  const int dl_row = lane / kChunks;
-  const int dl_pos = lane % kChunks;
+  // The loads are buffer loads: the tile's first row is the descriptor's base, a lane's offset inside a row group (row
+  // l / kChunks, the chunk the swizzle maps to position l % kChunks) is one loop-invariant register per operand --
+  // the swizzle term does not depend on which of the wave's row groups it is -- and everything that changes from
+  // load to load (row group, k) is a scalar offset: no vector address arithmetic in the loop.
+  static_assert((kWaves * kRowsPerLoad / kRowsPerSweep) % kChunks == 0, "the swizzle must repeat from one row group of a wave to the next");
+  const int dl_row = wave * kRowsPerLoad + lane / kChunks;
+  const int dl_chunk = (lane % kChunks) ^ ((dl_row / kRowsPerSweep) % kChunks);
+  const uint32_t lane_offset_p = static_cast<uint32_t>(dl_row * a.ldp + dl_chunk * 8) * 2u;
+  const uint32_t lane_offset_q = static_cast<uint32_t>(dl_row * a.ldq + dl_chunk * 8) * 2u;
+  auto operand_rsrc = [](const __bf16* base, int64_t rows, int ld) {
+    const int64_t bytes = rows * ld * 2;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base), 0, static_cast<int>(bytes < 0x7fffffff ? bytes : 0x7fffffff), 0x00020000);
+  };
+  const __amdgpu_buffer_rsrc_t rsrc_p = operand_rsrc(P, a.M - row0, a.ldp);
+  const __amdgpu_buffer_rsrc_t rsrc_q = operand_rsrc(Q, a.N - col0, a.ldq);
+  typedef __attribute__((address_space(3))) void* LdsPtr;
   // One load at a time: a wave that issues several of these back to back stalls on the address queue, and its
   // MFMAs wait with it, so the main loop slips them in between MFMAs.
   auto load_p = [&](int k0, int stage, int i) {
     const int r0 = (i * kWaves + wave) * kRowsPerLoad;
-    const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
-    const __bf16* src = P + static_cast<int64_t>(r0 + dl_row) * a.ldp + k0 + chunk * 8;
-    __builtin_amdgcn_global_load_lds(src, smem + stage * kStageElems + r0 * BK, 16, 0, 0);
+    const int scalar_offset = (i * kWaves * kRowsPerLoad * a.ldp + k0) * 2;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_p, (LdsPtr)(smem + stage * kStageElems + r0 * BK), 16, lane_offset_p, scalar_offset, 0, 0);
   };
   auto load_q = [&](int k0, int stage, int i) {
     const int r0 = (i * kWaves + wave) * kRowsPerLoad;
-    const int chunk = dl_pos ^ (((r0 + dl_row) / kRowsPerSweep) % kChunks);
-    const __bf16* src = Q + static_cast<int64_t>(r0 + dl_row) * a.ldq + k0 + chunk * 8;
-    __builtin_amdgcn_global_load_lds(src, smem + stage * kStageElems + BM * BK + r0 * BK, 16, 0, 0);
+    const int scalar_offset = (i * kWaves * kRowsPerLoad * a.ldq + k0) * 2;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, (LdsPtr)(smem + stage * kStageElems + BM * BK + r0 * BK), 16, lane_offset_q, scalar_offset, 0, 0);
   };
   auto stream_p = [&](int k0, int stage) {
 #pragma unroll
@@ -179,39 +192,22 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
   // (A D tile fetched behind the main loop has to be staged through LDS, since its rows do not match the accumulator
   // layout, and picked up with 2-byte LDS reads: 5 of the 121 microseconds of a 256x256 tile with K = 4096.  The
   // fetch itself stays what it is wherever it sits: every CU wants its 128 KiB at the same moment.)
-  const bool start_from_d = whole && a.DT != nullptr;
+  // A whole tile takes its D operand on the way: D^T is the Q operand itself in both products that have one (X^T in
+  // the update product, the symmetric A in A A), and K spans the rows of C there, so the Q slabs with k in
+  // [row0, row0 + BM) hold D[k - row0][0 .. BN) of this tile as they pass through LDS.  The waves pick their values
+  // out of those slabs (see the slab loop) and add (beta / alpha) D to the accumulators, so that alpha * acc is
+  // alpha P Q^T + beta D with one rounding; nothing is fetched for D.  (Fetched behind the main loop the D tile
+  // cost a 256 x 256 tile with K = 4096 11 of its 121 microseconds: every CU wants its 128 KiB from HBM at the same
+  // moment, and the tile has to be staged through LDS because its rows do not match the accumulator layout.)
+  const bool d_in_slabs = whole && a.D != nullptr;
+  const float d_scale = d_in_slabs ? a.beta / a.alpha : 0.0f;
   f32x4 acc[TM][TN];
-  u32x2 d_raw[TM][TN];
-  if (start_from_d) {
-    const uint16_t* __restrict__ DT = static_cast<const uint16_t*>(a.DT);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int i = 0; i < TM; ++i)  // consecutive i: consecutive 32-byte pieces of the same rows of D^T
-        d_raw[i][j] = *reinterpret_cast<const u32x2*>(DT + static_cast<int64_t>(col0 + lcol + j * 16) * a.lddt + row0 + lrow + i * 16);
-  }
-  // (the values are turned into accumulators behind the first slab loads, so that the two fetches overlap)
-  auto start_accumulators = [&]() {
-    if (start_from_d) {
-      const float scale = a.beta / a.alpha;
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          acc[i][j][0] = scale * __uint_as_float(d_raw[i][j].x << 16);
-          acc[i][j][1] = scale * __uint_as_float(d_raw[i][j].x & 0xffff0000u);
-          acc[i][j][2] = scale * __uint_as_float(d_raw[i][j].y << 16);
-          acc[i][j][3] = scale * __uint_as_float(d_raw[i][j].y & 0xffff0000u);
-        }
-    } else {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
-    }
-  };
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
   // 16x16x32 MFMA operands: lane l supplies row l % 16 of its 16-row block and the 8 k values of chunk l / 16 of
   // the 32 wide step.  (At equal peak rate this shape draws less power than 32x32x16 on operands with random
@@ -251,8 +247,6 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       stream_p(k0_clamped(sidx), sidx);
       if (sidx + 1 < STAGES) stream_q(k0_clamped(sidx), sidx);  // the Q rows of the last one go out under the first MFMAs
     }
-    __builtin_amdgcn_sched_barrier(0);  // the slab loads are on their way before the D values are waited for
-    start_accumulators();
     constexpr int kAfterFirst = (STAGES - 2) * kLoadsPerSlab + kLoadsP;
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kAfterFirst & 0xF) | ((kAfterFirst >> 4) << 14));
     __syncthreads();
@@ -261,8 +255,6 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int i = 0; i < TMH; ++i) fa_lo[i] = *reinterpret_cast<const bf16x8*>(frag_p + off + i * 16 * BK);
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb0[j] = *reinterpret_cast<const bf16x8*>(frag_q + off + j * 16 * BK);
-  } else {
-    start_accumulators();
   }
   // One half step: the TMH x TN MFMAs on the fragments in hand (use_a for tile rows row0.., use_b), kReads LDS
   // reads (read(r), one behind each of the first MFMAs) and kLoads slab loads, interleaved instruction by
@@ -316,14 +308,57 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
               },
               loads_tag, load);
   };
+  // D values out of a Q slab (see d_in_slabs above).  Slab q of the BM / BK slabs that hold the tile's D rows carries
+  // the rows of kTilesPerSlab MFMA tile rows of the waves with wave_m == q / kSlabsPerWave; a lane's four rows of one
+  // column are four consecutive k of one slab row: one 64-bit LDS read per MFMA tile, in three batches at the starts
+  // of the slab's first three half steps (the values wait in registers for half a step, and all reads are back before
+  // the barrier that releases the stage).
+  constexpr int kTilesPerSlab = BK / 16;
+  constexpr int kSlabsPerWave = kWaveM / BK;
+  constexpr int kDSlabs = BM / BK;
+  constexpr int kDPairs = kTilesPerSlab * TN, kDBatches = 3, kDBatch = (kDPairs + kDBatches - 1) / kDBatches;
+  static_assert(kWaveM % BK == 0 && TM == kSlabsPerWave * kTilesPerSlab && kSteps == 2, "D slabs must divide over the waves and the half steps");
+  const int d_base = BM * BK + lcol * BK + 4 * ((lane >> 4) & 1);  // slab row lcol (+ 16 j), first or second half of a chunk
+  const int d_swizzle = (lcol / kRowsPerSweep) % kChunks;          // the same for lcol + 16 j
+  u32x2 d_vals[kDBatch];
+  auto d_read = [&](int stage, int batch) {
+#pragma unroll
+    for (int n = 0; n < kDBatch; ++n) {
+      const int pair = batch * kDBatch + n, ii = pair / TN, j = pair % TN;
+      if (pair >= kDPairs) break;
+      const int chunk = (2 * ii + (lane >> 5)) ^ d_swizzle;
+      d_vals[n] = *reinterpret_cast<const u32x2*>(smem + stage * kStageElems + d_base + j * 16 * BK + (chunk << 3));
+    }
+  };
+  auto d_add = [&](auto qq_tag, int batch, float scale) {
+    constexpr int kFirstTile = decltype(qq_tag)::value * kTilesPerSlab;
+#pragma unroll
+    for (int n = 0; n < kDBatch; ++n) {
+      const int pair = batch * kDBatch + n, i = kFirstTile + pair / TN, j = pair % TN;
+      if (pair >= kDPairs) break;
+      acc[i][j][0] += scale * __uint_as_float(d_vals[n].x << 16);
+      acc[i][j][1] += scale * __uint_as_float(d_vals[n].x & 0xffff0000u);
+      acc[i][j][2] += scale * __uint_as_float(d_vals[n].y << 16);
+      acc[i][j][3] += scale * __uint_as_float(d_vals[n].y & 0xffff0000u);
+    }
+  };
   int stage = 0;
-  for (int it = 0; it < n_slabs; ++it) {
+  // One slab.  d_tag: -1, or which of the tile's D slabs this one is.
+  auto slab = [&](int it, auto d_tag) {
+    constexpr int kD = decltype(d_tag)::value;
+    constexpr int kOwner = kD < 0 ? 0 : kD / kSlabsPerWave;
+    using Part = std::integral_constant<int, kD < 0 ? 0 : kD % kSlabsPerWave>;
+    const float scale = (kD >= 0 && wave_m == kOwner) ? d_scale : 0.0f;  // the other waves add zero times a finite value
     const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
     const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
 #pragma unroll
     for (int kk = 0; kk < kSteps; kk += 2) {
       __builtin_amdgcn_s_waitcnt(kWaitLds);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kD >= 0) {
+        d_read(stage, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (kk == 0) {
         // second half of the refill of the stage the previous slab's barrier released (its P rows went out there)
         const int k0 = k0_clamped(it - 1 + STAGES);
@@ -333,9 +368,19 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
       }
       __builtin_amdgcn_s_waitcnt(kWaitLds);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kD >= 0) {
+        d_add(Part{}, 0, scale);
+        d_read(stage, 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       second_half(fb0, fb1, stage, kk + 1, Zero{}, [](int) {});
       __builtin_amdgcn_s_waitcnt(kWaitLds);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kD >= 0) {
+        d_add(Part{}, 1, scale);
+        d_read(stage, 2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       first_half(fb1, stage, kk + 1, Zero{}, [](int) {});
       if (kk + 2 < kSteps) {
         __builtin_amdgcn_s_waitcnt(kWaitLds);
@@ -347,11 +392,30 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
         __builtin_amdgcn_s_waitcnt(kWaitNextSlab);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kD >= 0) {
+          d_add(Part{}, 2, scale);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         const int k0 = k0_clamped(it + STAGES);
         second_half(fb1, fb0, next_stage, 0, std::integral_constant<int, kLoadsP>{}, [&](int l) { load_p(k0, stage, l); });
       }
     }
     stage = next_stage;
+  };
+  using NoD = std::integral_constant<int, -1>;
+  if (d_in_slabs) {
+    // the slabs with k in [row0, row0 + BM) are peeled out of the walk (whole tiles walk all of K from slab 0)
+    const int first_d = row0 / BK;
+    for (int it = 0; it < first_d; ++it) slab(it, NoD{});
+    auto d_slabs = [&](auto&& self, auto q_tag) -> void {
+      constexpr int kQ = decltype(q_tag)::value;
+      slab(first_d + kQ, q_tag);
+      if constexpr (kQ + 1 < kDSlabs) self(self, std::integral_constant<int, kQ + 1>{});
+    };
+    d_slabs(d_slabs, Zero{});
+    for (int it = first_d + kDSlabs; it < n_slabs; ++it) slab(it, NoD{});
+  } else {
+    for (int it = 0; it < n_slabs; ++it) slab(it, NoD{});
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // the loads past the end of the walk have landed too; LDS is free
 
@@ -620,15 +684,16 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   if ((a.ldc % 8) || reinterpret_cast<uintptr_t>(a.C) % 16 || (a.D && ((a.ldd % 8) || reinterpret_cast<uintptr_t>(a.D) % 16)) ||
       (a.CT && ((a.ldct % 8) || reinterpret_cast<uintptr_t>(a.CT) % 16)))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: C, D and the transposed output must be 16-byte aligned with leading dimensions multiple of 8");
-  if ((a.D != nullptr) != (a.DT != nullptr)) return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: D and its transpose come together");
-  if (a.DT && (a.lddt < a.M || (a.lddt % 4) || reinterpret_cast<uintptr_t>(a.DT) % 8 || a.alpha == 0.0f))
-    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: the transposed D needs alpha != 0, 8-byte alignment and a leading dimension >= M that is a multiple of 4");
+  if (a.D && (!a.d_transposed_is_q || a.K < a.M || a.alpha == 0.0f))
+    return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: a D operand needs D^T == Q (K >= M) and alpha != 0");
+  if (a.ldp > (1 << 22) || a.ldq > (1 << 22)) return fail(MFSDP_ERR_UNSUPPORTED, "gemm_nt_bf16: leading dimensions beyond 2^22 elements");
+  const GemmNtArgs& b = a;
   const GemmTuning tuning = tuning_snapshot();
   // Slabs of 32 (three to five deep) were measured too: each slab row is then half a 128-byte line, the vector
   // cache looks every line up twice, and the products run 15-25 % slower than with slabs of 64 two deep.
-  if (choose_variant(a, tuning) == 2)  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
-    return launch<128, 128, 2, 2, 64, 2, 2>(a, scratch, tuning, stream);
-  return launch<256, 256, 2, 4, 64, 2, 1>(a, scratch, tuning, stream);  // 256x256 tile, 8 waves of 128x64, one workgroup per CU
+  if (choose_variant(b, tuning) == 2)  // 128x128 tile, 4 waves of 64x64, two workgroups per CU
+    return launch<128, 128, 2, 2, 64, 2, 2>(b, scratch, tuning, stream);
+  return launch<256, 256, 2, 4, 64, 2, 1>(b, scratch, tuning, stream);  // 256x256 tile, 8 waves of 128x64, one workgroup per CU
 }
 
 }  // namespace mfsdp
