@@ -284,10 +284,8 @@ int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_buf, int dt
  * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
  * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU; for the symmetric products also 3, the default:
  * whichever of the two fills the CUs better for the size at hand), the tile rows the general products walk together
- * (default 4), K-splitting of the last partial round of tiles on (1) / off (2), and its cap;
- * stagger >= 0 sets the K-walk start offset, in 64-element slabs, between consecutive tiles. */
-void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder,
-                           int max_splits, int stagger);
+ * (default 4), K-splitting of the last partial round of tiles on (1) / off (2), and its cap. */
+void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder, int max_splits);
 
 /* ------------------------------------------------------------------ AdamW */
 

@@ -187,13 +187,12 @@ extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf
 }
 
 extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder,
-                                      int max_splits, int stagger) {
+                                      int max_splits) {
   GemmTuning t = get_gemm_tuning();
   if (general_variant > 0) t.general_variant = general_variant;
   if (symmetric_variant > 0) t.symmetric_variant = symmetric_variant;
   if (group_m > 0) t.group_m = group_m;
   if (split_remainder > 0) t.split_remainder = split_remainder == 1;
   if (max_splits > 0) t.max_splits = max_splits;
-  if (stagger >= 0) t.stagger = stagger;
   set_gemm_tuning(t);
 }

@@ -44,7 +44,6 @@ struct GemmTuning {
   int group_m = 4;            // general products: tile rows walked together (the workgroups of one XCD share their P panels)
   int split_remainder = 1;    // split the tiles of the last partial round along K
   int max_splits = 16;
-  int stagger = 0;            // K-walk start offset (slabs) between consecutive tiles; 0 = none
 };
 void set_gemm_tuning(const GemmTuning& tuning);
 GemmTuning get_gemm_tuning();

@@ -217,11 +217,11 @@ def test_symmetric_tile_variants_forced(shape, variant):
 
     u = normal_flat(shape[0] * shape[1], 1e-3, 9, torch.float32).view(shape)
     want = OO.newton_schulz(u).float()
-    _lib.lib().mfsdp_set_muon_tuning(0, variant, 0, 0, 0, -1)
+    _lib.lib().mfsdp_set_muon_tuning(0, variant, 0, 0, 0)
     try:
         have = F.newton_schulz(u.to(DEV)).float().cpu()
     finally:
-        _lib.lib().mfsdp_set_muon_tuning(0, 3, 0, 0, 0, -1)
+        _lib.lib().mfsdp_set_muon_tuning(0, 3, 0, 0, 0)
     assert rel_fro(have, want) < MUON_TOL
 
 
