@@ -208,20 +208,23 @@ def test_hidden4096_matrices_side_by_side_against_torch_muon():
     assert rel_fro(p_dev[0].cpu() - p0[0], p_ref - p0[0]) < MUON_TOL
 
 
+@pytest.mark.parametrize("general", [1, 2])
 @pytest.mark.parametrize("variant", [1, 2])
-@pytest.mark.parametrize("shape", [(512, 768), (768, 512), (1024, 1024)])
-def test_symmetric_tile_variants_forced(shape, variant):
-    """Both tilings of the symmetric products (1: 256 x 256 with mirrored store, 2: 128 x 128) forced on small
-    shapes, where the CPU oracle is cheap; the default chooser is restored afterwards."""
+@pytest.mark.parametrize("shape", [(512, 768), (768, 512), (1024, 1024), (256, 1280)])
+def test_tile_variants_forced(shape, variant, general):
+    """Both tilings (1: 256 x 256, 2: 128 x 128) forced for the symmetric products (mirrored store, D picked out of
+    the slabs of the symmetric operand) and for the general product (D picked out of the X^T slabs, both orientations
+    written) on small shapes, where the CPU oracle is cheap -- one to four tile rows, so that the slabs that carry a
+    tile's D values sit first, in the middle and last in its K walk; the default chooser is restored afterwards."""
     from matrix_fsdp_amd import _lib
 
     u = normal_flat(shape[0] * shape[1], 1e-3, 9, torch.float32).view(shape)
     want = OO.newton_schulz(u).float()
-    _lib.lib().mfsdp_set_muon_tuning(0, variant, 0, 0, 0)
+    _lib.lib().mfsdp_set_muon_tuning(general, variant, 0, 0, 0)
     try:
         have = F.newton_schulz(u.to(DEV)).float().cpu()
     finally:
-        _lib.lib().mfsdp_set_muon_tuning(0, 3, 0, 0, 0)
+        _lib.lib().mfsdp_set_muon_tuning(1, 3, 0, 0, 0)
     assert rel_fro(have, want) < MUON_TOL
 
 
