@@ -326,6 +326,17 @@ def main() -> int:
             flops += fl
             t, _ = time_launches(torch, lambda: F.muon_step(p, g, buf, workspace=ws, **kw), 20, 5)
             per_matrix[f"{shape[0]}x{shape[1]}"] = {"ms": round(t, 4), "TFLOPs": round(fl / (t * 1e-3) / 1e12, 1)}
+        # the optimizer the reference builds for these parameters (torch.optim.Muon: hipBLASLt products, full GEMMs), same
+        # GPU, same hyper-parameters, on copies of the tensors: the reference's own execution of this step, for scale
+        torch_ms = None
+        if hasattr(torch.optim, "Muon"):
+            t_params = [torch.nn.Parameter(p.clone()) for p, _, _ in mats]
+            t_opt = torch.optim.Muon(t_params, lr=kw["lr"], weight_decay=kw["weight_decay"], momentum=kw["momentum"], nesterov=kw["nesterov"],
+                                     ns_coefficients=NS_COEFFS, eps=kw["eps"], ns_steps=kw["ns_steps"])
+            for tp, (_, g, _) in zip(t_params, mats):
+                tp.grad = g.clone()
+            torch_ms, _ = time_launches(torch, t_opt.step, 10, 3)
+            del t_opt, t_params
         tflops = flops / (med * 1e-3) / 1e12
         legs["muon_hidden4096"] = {
             "ms_per_step": round(med, 4),
@@ -338,6 +349,8 @@ def main() -> int:
             "dtype_variant": "fp32 params / momentum, bf16-valued fp32 grads",
             "per_matrix": per_matrix,
         }
+        if torch_ms is not None:
+            legs["muon_hidden4096"]["torch_optim_muon_same_gpu"] = {"ms_per_step": round(torch_ms, 4), "ns_TFLOPs_reference_flop_count": round(flops / (torch_ms * 1e-3) / 1e12, 1)}
         result["muon_ns_TFLOPs"] = round(tflops, 1)
         result["muon_ms_per_step"] = round(med, 4)
         executed = sum(int(_lib.lib().mfsdp_muon_executed_flops(sh[0], sh[1], 5, _lib.MUON_SHARED_MACHINE)) for sh in MUON_HIDDEN4096_SHAPES)
