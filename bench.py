@@ -254,7 +254,30 @@ def main() -> int:
             "mfsdp_hbm_probe; the equal mix is the rate at which half the bytes move at the read-only and half at the write-only rate",
         }
         result["roofline"]["frac_of_plain_copy"] = round(achieved / legs["hbm_ceiling_one_layer_buffer"]["plain_copy_GBps"], 4)
-        del a_buf, b_buf, sink
+        # what the segment programs stand in for: the reference's per-segment slice copies (flat_buffer.py:1304-1316), on this
+        # GPU, for ONE rank's shard of one layer buffer (a quarter of a pack), once after a warm-up pass
+        rank_segments = plan.rank_segments[0]
+        shard = torch.empty(plan.max_shard_size, dtype=torch.bfloat16, device=dev)
+
+        def slice_copy_loop():
+            for seg in rank_segments:
+                shard[seg.local_start : seg.local_start + seg.numel].copy_(a_buf[seg.global_start : seg.global_start + seg.numel])
+
+        slice_copy_loop()
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        slice_copy_loop()
+        torch.cuda.synchronize(dev)
+        t_loop = time.perf_counter() - t0
+        loop_bytes = 2 * 2 * sum(seg.numel for seg in rank_segments)
+        legs["reference_slice_copy_loop_same_gpu"] = {
+            "segments": len(rank_segments),
+            "ms_one_rank_shard": round(t_loop * 1e3, 2),
+            "GBps": round(loop_bytes / t_loop / 1e9, 2),
+            "note": "torch slice copy_ per layout segment, as the reference packs a rank's shard without its extension; rank 0 of one "
+            "hidden4096 layer buffer, wall time including the launches",
+        }
+        del a_buf, b_buf, sink, shard
         torch.cuda.empty_cache()
 
     if "rows" in want:
