@@ -62,6 +62,8 @@ def parse_args():
     ap.add_argument("--legs", default="ceiling,rows,muon,adamw,mixed",
                     help="comma list of the extra legs to run: ceiling (plain copy / read-only / write-only probes), rows (hidden2048 row split), muon, adamw, mixed")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
+    ap.add_argument("--hold-muon-seconds", type=float, default=0.0,
+                    help="after the Muon leg, keep stepping for this long (for sampling the clock beside it); reports the rate of that stretch")
     ap.add_argument("--no-launch-events", action="store_true", help="no HIP events inside the timed region (launch time from the wall clock)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain Tensor.copy_ of 1 GiB (a copy kernel of known size, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -376,6 +378,15 @@ def main() -> int:
             legs["muon_hidden4096"]["torch_optim_muon_same_gpu"] = {"ms_per_step": round(torch_ms, 4), "ns_TFLOPs_reference_flop_count": round(flops / (torch_ms * 1e-3) / 1e12, 1)}
         result["muon_ns_TFLOPs"] = round(tflops, 1)
         result["muon_ms_per_step"] = round(med, 4)
+        if args.hold_muon_seconds > 0:
+            t_hold, n_hold = time.perf_counter(), 0
+            while time.perf_counter() - t_hold < args.hold_muon_seconds:
+                for _ in range(20):
+                    muon_all()
+                torch.cuda.synchronize(dev)
+                n_hold += 20
+            held = (time.perf_counter() - t_hold) / n_hold * 1e3
+            legs["muon_hidden4096"]["held"] = {"seconds": args.hold_muon_seconds, "ms_per_step": round(held, 4), "ns_TFLOPs_reference_flop_count": round(flops / (held * 1e-3) / 1e12, 1)}
         executed = sum(int(_lib.lib().mfsdp_muon_executed_flops(sh[0], sh[1], 5, _lib.MUON_SHARED_MACHINE)) for sh in MUON_HIDDEN4096_SHAPES)
         tflops_executed = executed / (med * 1e-3) / 1e12
         legs["muon_hidden4096"]["ns_TFLOPs_executed"] = round(tflops_executed, 1)
