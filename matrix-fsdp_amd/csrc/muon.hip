@@ -12,6 +12,7 @@
 #include "muon_gemm.h"
 
 #include <algorithm>
+#include <cmath>
 
 namespace mfsdp {
 namespace {
@@ -81,13 +82,19 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     g.ldp = w.np; g.ldq = w.np; g.ldd = 0; g.ldc = w.mp; g.ldct = 0;
     g.alpha = 1.0f; g.beta = 0.0f; g.symmetric = 1; g.shared = shared;
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
-    g = GemmNtArgs{};
-    g.P = w.A; g.Q = w.A; g.D = w.A; g.C = w.B; g.CT = nullptr;
-    g.d_transposed_is_q = 1;  // A is symmetric
-    g.M = w.mp; g.N = w.mp; g.K = w.mp;
-    g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.mp; g.ldc = w.mp; g.ldct = 0;
-    g.alpha = c; g.beta = b; g.symmetric = 1; g.shared = shared;
-    if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
+    if (c == 0.0f) {
+      // addmm with alpha = 0 leaves beta * A (the product is not formed at all, torch/optim/_muon.py:61 with a
+      // quadratic polynomial); the GEMM's D path needs alpha != 0 (it adds (beta / alpha) D to the accumulators)
+      if (int rc = muon_scale_bf16(w.B, w.A, static_cast<int64_t>(w.mp) * w.mp, b, stream)) return rc;
+    } else {
+      g = GemmNtArgs{};
+      g.P = w.A; g.Q = w.A; g.D = w.A; g.C = w.B; g.CT = nullptr;
+      g.d_transposed_is_q = 1;  // A is symmetric
+      g.M = w.mp; g.N = w.mp; g.K = w.mp;
+      g.ldp = w.mp; g.ldq = w.mp; g.ldd = w.mp; g.ldc = w.mp; g.ldct = 0;
+      g.alpha = c; g.beta = b; g.symmetric = 1; g.shared = shared;
+      if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
+    }
     g = GemmNtArgs{};
     g.P = w.B; g.Q = w.XT[cur]; g.D = w.X[cur]; g.C = w.X[nxt]; g.CT = w.XT[nxt];
     g.d_transposed_is_q = 1;  // Q = X^T
@@ -106,7 +113,10 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
   return MFSDP_OK;
 }
 
-int check_common(int64_t rows, int64_t cols, int steps, const void* workspace, int64_t workspace_bytes, Workspace* w) {
+int check_common(int64_t rows, int64_t cols, float a, float b, float c, int steps, const void* workspace, int64_t workspace_bytes, Workspace* w) {
+  // everything that can be refused is refused here, before the first kernel is enqueued (a step must not be left half applied)
+  if (!std::isfinite(a) || !std::isfinite(b) || !std::isfinite(c) || (c != 0.0f && !std::isfinite(b / c)))
+    return fail(MFSDP_ERR_INVALID, "Newton-Schulz coefficients must be finite (and b / c representable), got (%g, %g, %g)", a, b, c);
   if (steps < 0 || steps >= 100) return fail(MFSDP_ERR_INVALID, "Number of steps must be less than 100 for computational efficiency");
   if (!plan_workspace(rows, cols, const_cast<void*>(workspace), w))
     return fail(MFSDP_ERR_INVALID, "Input tensor gradient must be a 2D matrix with positive sizes, got %lld x %lld",
@@ -142,7 +152,7 @@ extern "C" int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int ste
 extern "C" int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t rows, int64_t cols, float a, float b, float c,
                                    int steps, float eps, void* out_bf16, void* workspace, int64_t workspace_bytes, void* stream) {
   Workspace w;
-  if (int rc = check_common(rows, cols, steps, workspace, workspace_bytes, &w)) return rc;
+  if (int rc = check_common(rows, cols, a, b, c, steps, workspace, workspace_bytes, &w)) return rc;
   if (update_dtype != MFSDP_F32 && update_dtype != MFSDP_BF16) return fail(MFSDP_ERR_INVALID, "update dtype must be f32 or bf16");
   if (!update || !out_bf16) return fail(MFSDP_ERR_INVALID, "null tensor pointer");
   hipStream_t s = as_stream(stream);
@@ -158,7 +168,7 @@ extern "C" int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_
                                   double weight_decay, double momentum, int nesterov, float a, float b, float c, int steps, float eps,
                                   double adjusted_lr, int flags, void* workspace, int64_t workspace_bytes, void* stream) {
   Workspace w;
-  if (int rc = check_common(rows, cols, steps, workspace, workspace_bytes, &w)) return rc;
+  if (int rc = check_common(rows, cols, a, b, c, steps, workspace, workspace_bytes, &w)) return rc;
   if (dtype != MFSDP_F32 && dtype != MFSDP_BF16) return fail(MFSDP_ERR_INVALID, "dtype must be f32 or bf16");
   if (!param || !grad || !momentum_buf) return fail(MFSDP_ERR_INVALID, "null tensor pointer");
   if (!(lr >= 0.0)) return fail(MFSDP_ERR_INVALID, "Learning rate should be >= 0 but is: %g", lr);

@@ -21,6 +21,8 @@ int muon_scale_transpose(const void* xraw, int rows, int cols, const float* scal
 // param <- round(round(param*decay) + neg_lr*ortho), ortho bf16 with leading dimension ldo
 int muon_apply(void* param, int dtype, const void* ortho, int rows, int cols, int ldo, float decay, float neg_lr,
                hipStream_t stream);
+// out <- bf16(scale * in) over numel contiguous bf16 (whole 16-byte groups)
+int muon_scale_bf16(void* out, const void* in, int64_t numel, float scale, hipStream_t stream);
 // out[rows x cols] contiguous bf16 <- ortho (leading dimension ldo)
 int muon_extract(void* out, const void* ortho, int rows, int cols, int ldo, hipStream_t stream);
 

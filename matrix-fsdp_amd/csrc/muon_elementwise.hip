@@ -63,6 +63,7 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // four consecutive elements at index 4*v (the caller guarantees the alignment)
 template <typename T>
@@ -234,6 +235,22 @@ extract_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ ortho, i
       out[static_cast<int64_t>(r) * cols + c] = ortho[static_cast<int64_t>(r) * ldo + c];
 }
 
+// out <- bf16(scale * in) over n contiguous bf16 (n a multiple of 8, both 16-byte aligned)
+__global__ void __launch_bounds__(kThreads)
+scale_bf16_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out, int64_t groups, float scale) {
+  for (int64_t g = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x; g < groups; g += static_cast<int64_t>(gridDim.x) * kThreads) {
+    const u32x4 v = in[g];
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t lo = f32_to_bf16(scale * bf16_to_f32(static_cast<uint16_t>(v[e])));
+      const uint32_t hi = f32_to_bf16(scale * bf16_to_f32(static_cast<uint16_t>(v[e] >> 16)));
+      r[e] = lo | (hi << 16);
+    }
+    out[g] = r;
+  }
+}
+
 int partial_blocks(int64_t numel) {
   const int64_t want = (numel + kThreads * 8 - 1) / (kThreads * 8);
   return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(want, kMuonMaxPartials)));
@@ -297,6 +314,16 @@ int muon_apply(void* param, int dtype, const void* ortho, int rows, int cols, in
   else
     hipLaunchKernelGGL((apply_kernel<uint16_t>), grid, dim3(kThreads), 0, stream, static_cast<uint16_t*>(param), o, rows, cols, ldo, col_quads, decay, neg_lr);
   MFSDP_CHECK_LAUNCH("apply_kernel");
+  return MFSDP_OK;
+}
+
+int muon_scale_bf16(void* out, const void* in, int64_t numel, float scale, hipStream_t stream) {
+  if (numel % 8 || reinterpret_cast<uintptr_t>(out) % 16 || reinterpret_cast<uintptr_t>(in) % 16)
+    return fail(MFSDP_ERR_INVALID, "muon_scale_bf16: whole 16-byte groups only");
+  const int64_t groups = numel / 8;
+  const int blocks = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>((groups + kThreads - 1) / kThreads, 65535)));
+  hipLaunchKernelGGL(scale_bf16_kernel, dim3(blocks), dim3(kThreads), 0, stream, static_cast<const u32x4*>(in), static_cast<u32x4*>(out), groups, scale);
+  MFSDP_CHECK_LAUNCH("scale_bf16_kernel");
   return MFSDP_OK;
 }
 

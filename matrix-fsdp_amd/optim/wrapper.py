@@ -6,8 +6,8 @@ Mirrors the Muon / AdamW wiring of matrix_fsdp/optim/wrapper.py
 :827-846) with the inner optimizers replaced by the HIP-backed ``Muon`` and
 ``FusedAdamW`` of this package.  The "units" handed in are ``MatrixFlatBuffer``
 objects (or a module carrying them as ``_matrix_fsdp_flat_buffers``); the
-scheduler / lifecycle arguments of the reference have no counterpart here and
-are rejected rather than silently ignored.
+prefetch-scheduler arguments of the reference have no counterpart on one
+device: they are accepted by name and dropped, anything else is a ``TypeError``.
 """
 from __future__ import annotations
 
@@ -134,6 +134,92 @@ def classify_matrix_optimizer_params(module_or_units, *, default_matrix_optimize
     )
 
 
+_SCHEDULER_KWARG_NAMES = frozenset(
+    {
+        "max_unsharded_prefetch_units",
+        "max_forward_prefetch_units",
+        "max_backward_prefetch_units",
+        "backward_prefetch_timing",
+        "prefetch_policy",
+        "max_cached_full_param_buffers_per_key",
+        "max_cached_elastic_workspaces_per_key",
+        "max_active_full_param_buffers",
+        "max_active_full_param_numel",
+        "max_active_full_param_memory_mb",
+        "max_pending_backward_reduces",
+        "owner_backward_prefetch_with_pending_reduce",
+        "trim_cuda_cache",
+        "cuda_cache_trim_threshold_mb",
+        "scheduler_config",
+    }
+)
+
+
+class LazyMuon:
+    """``Muon`` built at the first ``step()`` (matrix_fsdp/optim/wrapper.py:615-684, ``_LazyMuonOptimizer``).
+
+    The reference delays ``torch.optim.Muon`` because an optimizer that allocates its momentum buffers up front can
+    push the first forward of a large model out of memory.  Until the first step this object answers with what an
+    optimizer without any state would: ``state == {}``, ``state_dict()["state"] == {}``, one parameter group holding
+    the constructor's keywords.  ``load_state_dict`` and ``add_param_group`` build the optimizer first."""
+
+    def __init__(self, params: Iterable[nn.Parameter], **kwargs: Any) -> None:
+        self.params = tuple(params)
+        self.kwargs = dict(kwargs)
+        self._built: Muon | None = None
+        self._pending_groups = [dict(self.kwargs, params=list(self.params))]
+
+    def _materialize(self) -> Muon:
+        if self._built is None:
+            with _without_auto_prepare():
+                self._built = Muon(self.params, **self.kwargs)
+        return self._built
+
+    @property
+    def param_groups(self) -> list[dict[str, Any]]:
+        return self._pending_groups if self._built is None else self._built.param_groups
+
+    @property
+    def state(self) -> dict[Any, Any]:
+        return {} if self._built is None else self._built.state
+
+    @property
+    def defaults(self) -> dict[str, Any]:
+        return dict(self.kwargs) if self._built is None else self._built.defaults
+
+    def step(self, closure=None):
+        built = self._materialize()
+        return built.step() if closure is None else built.step(closure=closure)
+
+    def zero_grad(self, set_to_none: bool = True) -> None:
+        if self._built is not None:
+            self._built.zero_grad(set_to_none=set_to_none)
+            return
+        for p in self.params:
+            if p.grad is None:
+                continue
+            if set_to_none:
+                p.grad = None
+            else:
+                p.grad.detach_()
+                p.grad.zero_()
+
+    def state_dict(self) -> dict[str, Any]:
+        if self._built is not None:
+            return self._built.state_dict()
+        groups = [dict({k: v for k, v in g.items() if k != "params"}, params=list(range(len(g["params"])))) for g in self._pending_groups]
+        return {"state": {}, "param_groups": groups}
+
+    def load_state_dict(self, state_dict: dict[str, Any]) -> None:
+        self._materialize().load_state_dict(state_dict)
+
+    def add_param_group(self, param_group: dict[str, Any]) -> None:
+        self._materialize().add_param_group(param_group)
+
+
+_LazyMuonOptimizer = LazyMuon  # the reference's name for it
+
+
 class MixedMuonAdamWOptimizer:
     """Muon on local full 2-D matrices, AdamW on everything else; the two inner
     optimizers stay separate objects.  Defaults follow the reference
@@ -152,14 +238,25 @@ class MixedMuonAdamWOptimizer:
         adamw_betas: tuple[float, float] = (0.9, 0.999),
         adamw_eps: float = 1e-8,
         adamw_weight_decay: float | None = None,
+        adamw_foreach: bool | None = None,
         muon_weight_decay: float | None = None,
         muon_momentum: float = 0.5,
         muon_ns_steps: int = 2,
         muon_adjust_lr_fn: str | None = DEFAULT_MUON_ADJUST_LR_FN,
+        lazy_muon_init: bool = False,
         flat_adamw_state: bool = False,
         flat_buffers: Iterable | None = None,
         fsdp_param_groups: Iterable | None = None,
+        **scheduler_kwargs: Any,
     ) -> None:
+        # The reference's constructor also takes its prefetch scheduler's settings (matrix_fsdp/optim/wrapper.py:384-399);
+        # one device has nothing to schedule, so exactly those names are accepted and dropped.  ``adamw_foreach`` picks
+        # between torch's two AdamW loops there; here AdamW is one fused launch per contiguous run either way.
+        unknown = sorted(set(scheduler_kwargs) - _SCHEDULER_KWARG_NAMES)
+        if unknown:
+            raise TypeError(f"MixedMuonAdamWOptimizer.__init__() got an unexpected keyword argument {unknown[0]!r}")
+        self.adamw_foreach = adamw_foreach
+        self.lazy_muon_init = bool(lazy_muon_init)
         self.fsdp_param_groups = list(fsdp_param_groups or ())
         self.muon_params = tuple(p for p in muon_params if p.numel() > 0)
         self.adamw_params = tuple(p for p in adamw_params if p.numel() > 0)
@@ -175,14 +272,14 @@ class MixedMuonAdamWOptimizer:
 
     def _build(self, lr, weight_decay, muon_lr, adamw_lr, adamw_betas, adamw_eps, adamw_weight_decay, muon_weight_decay, muon_momentum, muon_ns_steps, muon_adjust_lr_fn) -> None:
         if self.muon_params:
-            self.muon = Muon(
-                self.muon_params,
+            muon_kwargs = dict(
                 lr=lr if muon_lr is None else muon_lr,
                 momentum=muon_momentum,
                 ns_steps=muon_ns_steps,
                 weight_decay=weight_decay if muon_weight_decay is None else muon_weight_decay,
                 adjust_lr_fn=muon_adjust_lr_fn,
             )
+            self.muon = LazyMuon(self.muon_params, **muon_kwargs) if self.lazy_muon_init else Muon(self.muon_params, **muon_kwargs)
         if self.adamw_params:
             self.adamw = FusedAdamW(
                 self.adamw_params,
@@ -455,27 +552,6 @@ def _local_params(module_or_units) -> list[nn.Parameter]:
                 seen.add(id(p))
                 params.append(p)
     return params
-
-
-_SCHEDULER_KWARG_NAMES = frozenset(
-    {
-        "max_unsharded_prefetch_units",
-        "max_forward_prefetch_units",
-        "max_backward_prefetch_units",
-        "backward_prefetch_timing",
-        "prefetch_policy",
-        "max_cached_full_param_buffers_per_key",
-        "max_cached_elastic_workspaces_per_key",
-        "max_active_full_param_buffers",
-        "max_active_full_param_numel",
-        "max_active_full_param_memory_mb",
-        "max_pending_backward_reduces",
-        "owner_backward_prefetch_with_pending_reduce",
-        "trim_cuda_cache",
-        "cuda_cache_trim_threshold_mb",
-        "scheduler_config",
-    }
-)
 
 
 def configure_optimizer(module_or_units, optimizer: str | MatrixOptimizerConfig = "adamw", **kwargs: Any):

@@ -494,3 +494,41 @@ def test_bench_refuses_more_than_one_gpu_and_the_product_has_no_cpu_path():
     params = list(managed_params_from_module(torch.nn.Linear(4, 4)))
     with pytest.raises(RuntimeError, match="HIP device"):
         MatrixFlatBuffer(params, contiguous_even_plan(params[-1].end, 2), rank=0)
+
+
+def test_mixed_optimizer_constructor_surface_of_the_reference():
+    """Construction only (no step, so no device): the three cases of test/fsdp/test_bench_fsdp2_compare.py:406-424
+    and the keyword set of matrix_fsdp/optim/wrapper.py:353-400."""
+    from matrix_fsdp_amd.optim.wrapper import DEFAULT_MUON_ADJUST_LR_FN, MixedMuonAdamWOptimizer, _LazyMuonOptimizer
+
+    matrix = torch.nn.Parameter(torch.ones(4, 4))
+    vector = torch.nn.Parameter(torch.ones(4))
+    optimizer = MixedMuonAdamWOptimizer([matrix], [])
+    assert DEFAULT_MUON_ADJUST_LR_FN == "match_rms_adamw"
+    assert optimizer.muon is not None and optimizer.muon.param_groups[0]["adjust_lr_fn"] == DEFAULT_MUON_ADJUST_LR_FN
+    lazy = MixedMuonAdamWOptimizer([matrix], [vector], lazy_muon_init=True)
+    assert lazy.muon.state == {} and lazy.state == {}
+    assert lazy.muon.state_dict()["state"] == {}
+    assert lazy.muon.param_groups[0]["adjust_lr_fn"] == DEFAULT_MUON_ADJUST_LR_FN
+    assert isinstance(lazy.muon, _LazyMuonOptimizer) and lazy.muon.defaults["momentum"] == 0.5 and lazy.muon.defaults["ns_steps"] == 2
+    matrix.grad = torch.ones(4, 4)
+    lazy.zero_grad()
+    assert matrix.grad is None and lazy.muon.state == {}
+    matrix.grad = torch.ones(4, 4)
+    lazy.muon.zero_grad(set_to_none=False)
+    assert float(matrix.grad.abs().sum()) == 0.0
+    every_reference_keyword = dict(
+        lr=1e-3, weight_decay=0.01, muon_lr=None, adamw_lr=None, adamw_betas=(0.9, 0.999), adamw_eps=1e-8, adamw_weight_decay=None,
+        adamw_foreach=None, muon_weight_decay=None, muon_momentum=0.5, muon_ns_steps=2, muon_adjust_lr_fn="match_rms_adamw",
+        lazy_muon_init=False, fsdp_param_groups=None, max_unsharded_prefetch_units=None, max_forward_prefetch_units=None,
+        max_backward_prefetch_units=None, backward_prefetch_timing="pre_backward", prefetch_policy="static",
+        max_cached_full_param_buffers_per_key=0, max_cached_elastic_workspaces_per_key=0, max_active_full_param_buffers=None,
+        max_active_full_param_numel=None, max_active_full_param_memory_mb=None, max_pending_backward_reduces=1,
+        owner_backward_prefetch_with_pending_reduce="auto", trim_cuda_cache=False, cuda_cache_trim_threshold_mb=1024.0,
+        flat_adamw_state=False, scheduler_config=None,
+    )
+    MixedMuonAdamWOptimizer([matrix], [vector], group_summaries=(), **every_reference_keyword)
+    with pytest.raises(TypeError, match="unexpected keyword argument 'momentum'"):
+        MixedMuonAdamWOptimizer([matrix], [], momentum=0.9)
+    with pytest.raises(RuntimeError, match="at least one non-empty parameter"):
+        MixedMuonAdamWOptimizer([], [])

@@ -57,6 +57,36 @@ def test_newton_schulz_singular_values_land_near_one():
     assert sv.max() < 1.3 and sv.min() > 0.3
 
 
+@pytest.mark.parametrize("coefficients", [(1.5, -0.5, 0.0), (2.0, -1.5, 0.5), (0.0, 1.0, 1.0)])
+def test_newton_schulz_other_polynomials(coefficients):
+    """torch.optim.Muon takes any three coefficients; with c = 0 (the cubic iteration) addmm leaves b * A, with a = 0
+    the update product has no X term."""
+    for shape in ((256, 256), (300, 520), (512, 256)):
+        u = make(shape, 17)
+        want = O.newton_schulz(u, coefficients=coefficients, steps=3)
+        have = F.newton_schulz(u.to(DEV), ns_coefficients=coefficients, ns_steps=3)
+        assert rel_fro(have, want) < MUON_TOL, (shape, coefficients)
+    p, g, buf = make((256, 384), 18, 0.02), make((256, 384), 19).bfloat16().float(), make((256, 384), 20)
+    p_dev, buf_dev = p.to(DEV), buf.to(DEV)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    F.muon_step(p_dev, g.to(DEV), buf_dev, ns_coefficients=coefficients, ns_steps=3, **kw)
+    p_ref, buf_ref = p.clone(), buf.clone()
+    O.muon_step(p_ref, g, buf_ref, coefficients=coefficients, steps=3, **kw)
+    assert rel_fro(p_dev.cpu() - p, p_ref - p) < MUON_TOL
+
+
+def test_non_finite_coefficients_are_refused_before_anything_runs():
+    p, g, buf = make((64, 64), 21, 0.02).to(DEV), make((64, 64), 22).to(DEV), make((64, 64), 23).to(DEV)
+    before = (p.clone(), buf.clone())
+    for bad in ((float("nan"), -4.775, 2.0315), (3.4445, float("inf"), 2.0315), (3.4445, -4.775, 1e-45)):
+        with pytest.raises(RuntimeError, match="coefficients must be finite"):
+            F.muon_step(p, g, buf, lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True, ns_coefficients=bad)
+        with pytest.raises(RuntimeError, match="coefficients must be finite"):
+            F.newton_schulz(g, ns_coefficients=bad)
+    torch.cuda.synchronize()
+    assert torch.equal(p, before[0]) and torch.equal(buf, before[1])  # the momentum buffer was not touched
+
+
 def test_zero_update_stays_zero():
     have = F.newton_schulz(torch.zeros(64, 128, device=DEV))
     assert torch.count_nonzero(have) == 0

@@ -261,3 +261,49 @@ def test_hip_optimizers_are_torch_optimizers_of_the_same_kind():
     flat.step()
     first, second = (flat.state[p]["exp_avg"] for p in list(model.parameters())[:2])
     assert second.data_ptr() == first.data_ptr() + first.numel() * 4
+
+
+def test_mixed_optimizer_takes_the_reference_constructor_and_delays_muon_state():
+    """test/fsdp/test_bench_fsdp2_compare.py:406-424 and the construction of bench_fsdp2_compare.py:2648:
+    ``MixedMuonAdamWOptimizer(muon_params, adamw_params, lazy_muon_init=True)`` holds no state before the first step,
+    and steps like the eager optimizer afterwards."""
+    from matrix_fsdp_amd.optim.wrapper import DEFAULT_MUON_ADJUST_LR_FN, LazyMuon
+
+    matrix = nn.Parameter(torch.ones(4, 4, device=DEV))
+    eager = MixedMuonAdamWOptimizer([matrix], [])
+    assert DEFAULT_MUON_ADJUST_LR_FN == "match_rms_adamw"
+    assert eager.muon is not None and eager.muon.param_groups[0]["adjust_lr_fn"] == DEFAULT_MUON_ADJUST_LR_FN
+    lazy = MixedMuonAdamWOptimizer([matrix], [], lazy_muon_init=True)
+    assert lazy.state == {}
+    assert lazy.muon.state_dict()["state"] == {}
+    assert lazy.muon.param_groups[0]["adjust_lr_fn"] == DEFAULT_MUON_ADJUST_LR_FN
+    assert isinstance(lazy.muon, LazyMuon) and lazy.muon.state_dict()["param_groups"][0]["params"] == [0]
+
+    # the bench's construction: every 2-D parameter to Muon, the rest to AdamW, built lazily
+    gen = torch.Generator().manual_seed(11)
+    shapes = [(128, 256), (256,), (256, 128), (128,)]
+    params = [nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(DEV)) for s in shapes]
+    twins = [nn.Parameter(p.detach().clone()) for p in params]
+    split = lambda ps: ([p for p in ps if p.ndim == 2 and p.numel() > 0], [p for p in ps if p.ndim != 2 and p.numel() > 0])
+    opt = MixedMuonAdamWOptimizer(*split(params), lazy_muon_init=True, adamw_foreach=False, max_forward_prefetch_units=2,
+                                  prefetch_policy="static", scheduler_config=None, trim_cuda_cache=False)
+    ref = MixedMuonAdamWOptimizer(*split(twins))
+    assert opt.state == {} and opt.defaults["muon"] == {k: v for k, v in ref.defaults["muon"].items() if k in opt.defaults["muon"]}
+    opt.zero_grad()  # nothing to clear yet, and nothing gets built by it
+    assert opt.muon.state == {}
+    for step in range(2):
+        for p, t in zip(params, twins):
+            g = (torch.randn(p.shape, generator=gen) * 1e-3).to(DEV)
+            p.grad, t.grad = g.clone(), g.clone()
+        opt.step()
+        ref.step()
+        for p, t in zip(params, twins):
+            assert torch.equal(p.detach(), t.detach())  # same kernels, same order: bit-identical to the eager construction
+    assert set(opt.muon.state[params[0]]) == {"momentum_buffer"}
+    assert opt.state_dict()["muon"]["state"].keys() == ref.state_dict()["muon"]["state"].keys()
+    opt.load_state_dict(ref.state_dict())
+    fresh = MixedMuonAdamWOptimizer(*split(params), lazy_muon_init=True)
+    fresh.load_state_dict(ref.state_dict())  # loading builds the optimizer
+    assert torch.equal(fresh.muon.state[params[0]]["momentum_buffer"], ref.muon.state[twins[0]]["momentum_buffer"])
+    with pytest.raises(TypeError, match="unexpected keyword argument 'bogus'"):
+        MixedMuonAdamWOptimizer([matrix], [], bogus=1)
