@@ -179,6 +179,88 @@ def test_muon_step_full_size_parameter_delta(shape):
     assert torch.allclose(buf_dev.cpu(), buf_torch_gpu, rtol=1e-6, atol=1e-9)
 
 
+def _newton_schulz_unrounded(u: torch.Tensor, dtype: torch.dtype, steps: int = 5) -> torch.Tensor:
+    """The same iteration (torch/optim/_muon.py:31-70) with NO bf16 rounding anywhere: the input is the bf16-valued
+    update, every product and sum stays in ``dtype`` (fp32 or fp64).  What both bf16 executions approximate."""
+    a, b, c = OO.NS_COEFFICIENTS
+    x = u.bfloat16().to(dtype)
+    tall = x.size(0) > x.size(1)
+    if tall:
+        x = x.T
+    x = x / x.norm().clamp(min=OO.NS_EPS)
+    for _ in range(steps):
+        gram = x @ x.T
+        poly = b * gram + c * (gram @ gram)
+        x = a * x + poly @ x
+    return x.T if tall else x
+
+
+@pytest.mark.parametrize("shape", [(4096, 11008), (15360, 5120)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_newton_schulz_full_size_is_as_close_to_the_unrounded_iteration_as_torch(shape):
+    """A check the mathematics fixes: the iteration evaluated without any bf16 rounding (fp32 products on this GPU) is
+    what every bf16 execution approximates.  The HIP kernels must be as close to it as hipBLASLt's execution of the
+    reference's own function -- not merely equally far from a third chaotic trajectory."""
+    from torch.optim._muon import _zeropower_via_newtonschulz
+
+    prior = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        u = normal_flat(shape[0] * shape[1], 1e-3, 4, torch.float32).view(shape).to(DEV)
+        exact = _newton_schulz_unrounded(u, torch.float32).double()
+        have = F.newton_schulz(u).double()
+        torch_gpu = _zeropower_via_newtonschulz(u, OO.NS_COEFFICIENTS, 5, OO.NS_EPS).double()
+        ours, theirs = rel_fro(have, exact), rel_fro(torch_gpu, exact)
+        print(f"newton_schulz {shape}: HIP vs unrounded fp32 iteration {ours:.3e}, torch GPU vs the same {theirs:.3e}")
+        _report({"test": "newton_schulz_vs_unrounded_fp32", "shape": list(shape), "hip": ours, "torch_gpu": theirs})
+        assert ours <= 1.1 * theirs
+        # fp64 on a 512-row slice (every quantity of the iteration in double): the same statement against the exact
+        # polynomial of the slice's singular values, within reach of a double-precision evaluation
+        rows = u[:512] if shape[0] <= shape[1] else u[:, :512].T.contiguous()
+        exact64 = _newton_schulz_unrounded(rows, torch.float64)
+        ours64 = rel_fro(F.newton_schulz(rows.contiguous()).double(), exact64)
+        theirs64 = rel_fro(_zeropower_via_newtonschulz(rows.contiguous(), OO.NS_COEFFICIENTS, 5, OO.NS_EPS).double(), exact64)
+        print(f"newton_schulz 512-row slice of {shape}: HIP vs fp64 {ours64:.3e}, torch GPU vs fp64 {theirs64:.3e}")
+        _report({"test": "newton_schulz_slice_vs_fp64", "shape": list(rows.shape), "hip": ours64, "torch_gpu": theirs64})
+        assert ours64 <= 1.1 * theirs64
+        s_exact = torch.linalg.svdvals(exact64)
+        s_have = torch.linalg.svdvals(F.newton_schulz(rows.contiguous()).double())
+        assert float((s_have - s_exact).abs().max()) < 0.05  # the singular values follow the polynomial's
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prior
+
+
+@pytest.mark.parametrize("shape", [(12288, 4096), (5120, 13824)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_muon_step_full_size_all_bf16(shape):
+    """bf16 parameter, gradient and momentum buffer (the reference's local shard, gradient shard and
+    ``zeros_like(grad)`` state share one dtype, matrix_fsdp/runtime/flat_buffer.py:790-803) at full size against
+    ``torch.optim.Muon.step`` on this GPU.  The parameter moves by about lr * 0.2 * sqrt(max dim) * |O| ~ 1e-2 per
+    element next to values of 2e-2, so its bf16 rounding (2^-9 relative) is a visible part of the delta: the delta is
+    compared in units of that rounding, the orthogonalised update itself to the Muon tolerance."""
+    n = shape[0] * shape[1]
+    p0 = normal_flat(n, 0.02, 81, torch.bfloat16).view(shape)
+    g = normal_flat(n, 1e-3, 82, torch.bfloat16).view(shape)
+    buf0 = normal_flat(n, 1e-3, 83, torch.bfloat16).view(shape)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    p_dev, buf_dev = p0.to(DEV), buf0.to(DEV)
+    F.muon_step(p_dev, g.to(DEV), buf_dev, **kw)
+    p_t = torch.nn.Parameter(p0.to(DEV))
+    opt = torch.optim.Muon([p_t], **kw)
+    opt.state[p_t]["momentum_buffer"] = buf0.to(DEV)
+    p_t.grad = g.to(DEV)
+    opt.step()
+    delta, delta_torch = (p_dev.float() - p0.to(DEV).float()), (p_t.detach().float() - p0.to(DEV).float())
+    d = rel_fro(delta, delta_torch)
+    buf_equal = float((buf_dev == opt.state[p_t]["momentum_buffer"]).float().mean())
+    print(f"muon_step all-bf16 {shape}: delta vs torch on this GPU {d:.3e}, momentum buffers equal in {buf_equal:.6f} of the elements")
+    _report({"test": "muon_step_all_bf16", "shape": list(shape), "vs_torch_gpu": d, "momentum_equal_fraction": buf_equal})
+    assert buf_equal == 1.0  # lerp in fp32, rounded once: the same bits
+    # the orthogonalised updates agree to the Muon tolerance; what the two bf16 parameters add on top is at most one
+    # rounding step of the parameter each (2^-8 of |p| ~ 0.02 against a delta of ~ 1e-2 per element)
+    assert d < 5e-2
+    worst = float((p_dev.float() - p_t.detach().float()).abs().max())
+    assert worst <= 2.0 ** -8 * float(p0.abs().max()) * 2
+
+
 def test_hidden4096_matrices_side_by_side_against_torch_muon():
     """The three matrices of a hidden4096 layer updated at the same time on side streams (their symmetric products then
     run on 256 x 256 tiles): every parameter delta against ``torch.optim.Muon.step`` on this GPU and, for the square
