@@ -30,19 +30,24 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kUnroll = 4;
 constexpr int kTileVectors = kWave * kUnroll;
-constexpr int kCopyThreads = 256;
+constexpr int kCopyThreads = 64;  // one wavefront per workgroup
 constexpr int kWavesPerBlock = kCopyThreads / kWave;
 constexpr int kCountThreads = 256;
 constexpr int kCountPerThread = 4;
 constexpr int kBlockSegments = kCountThreads * kCountPerThread;  // segments whose tile counts one workgroup sums
 constexpr int kBlockShift = 10;
 static_assert(kBlockSegments == 1 << kBlockShift, "block of segments");
-// Consecutive tiles one bisection serves, and the workgroups per CU the balanced grid is capped at.  Measured on the
-// 21 250 row segments of a hidden4096 rank shard: (8 tiles, 4 per CU) 50 us, (4, 16) 48 us, (1, 64) 45 us, (1, 256) 59 us;
-// eight segments of 50 MB: 163, 176, 148, 155 us.  Many short-lived waves beat few long-lived ones, as in the other
-// copy kernels, until the empty workgroups of the upper-bound grid cost more than they hide.
+// Consecutive tiles one bisection serves, and the workgroups (of one wavefront each) per CU the balanced grid is capped at.
+// Measured on the 21 250 row segments of a hidden4096 rank shard, waves per CU = 4 x the figure given for workgroups of
+// four waves: (8 tiles, 16 waves per CU) 50 us, (4, 64) 48 us, (1, 256) 45 us, (1, 1024) 59 us; eight segments of 50 MB:
+// 163, 176, 148, 155 us.  Many short-lived waves beat few long-lived ones, as in the other copy kernels, until the empty
+// workgroups of the upper-bound grid cost more than they hide.  One wavefront per workgroup (dispatch in index order
+// sweeps neighbouring addresses) took the uniform shape from 5.4-5.7 to 5.8-6.0 TB/s on that shard, the level of the
+// compiled segment program; the balanced shape stays at 46 us there (its two count kernels are 9 us of that, and a
+// ballot search over the running counts in place of the bisection was slower still: 87 us -- the set-up of a wave that
+// moves 4 KiB is what costs), so it is the shape for layouts whose segment lengths differ widely, not for this one.
 constexpr int kChunkTiles = 1;
-constexpr int kBalancedBlocksPerCu = 64;
+constexpr int kBalancedBlocksPerCu = 256;
 constexpr int kMaxDevices = 64;
 
 // Scratch of the entry point that allocates nothing: the tile-count tables of up to kStaticMaxSegments segments.
@@ -203,12 +208,12 @@ __device__ __forceinline__ void copy_tiles_any(const Geometry& g, uint64_t tile_
 // ---- uniform launch shape: slot = (segment, j) with j < slots_per_segment, the tile count of the longest segment at
 // V = 16; the slot's wave moves tiles j, j + slots_per_segment, ... of its segment (more than one only when the
 // segment's addresses force a narrower vector).
-__global__ void __launch_bounds__(kCopyThreads)
+// One wavefront per workgroup: workgroups are dispatched in index order, so the waves in flight sweep neighbouring
+// addresses (as in the other copy kernels, small short-lived workgroups serve HBM best).
+__global__ void __launch_bounds__(kWave)
 segment_copy_uniform_kernel(SegmentCopyArgs a, uint64_t slots_per_segment, uint64_t n_slots) {
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWavesPerBlock;
-  const uint32_t wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keeps the metadata loads scalar
-  for (uint64_t slot = static_cast<uint64_t>(blockIdx.x) * kWavesPerBlock + wave_in_block; slot < n_slots; slot += n_waves) {
+  const uint32_t lane = threadIdx.x;
+  for (uint64_t slot = blockIdx.x; slot < n_slots; slot += gridDim.x) {
     const uint64_t s = slot / slots_per_segment;
     const uint64_t first = slot - s * slots_per_segment;
     const Geometry g = segment_geometry(a, static_cast<int64_t>(s));
@@ -359,9 +364,9 @@ int launch_balanced(const SegmentCopyArgs& a, uint64_t* tables, hipStream_t stre
   if (n_blocks > (int64_t{1} << 31) - 1) return fail(MFSDP_ERR_UNSUPPORTED, "%lld segments are beyond the grid", static_cast<long long>(a.n_segments));
   hipLaunchKernelGGL(segment_tile_count_kernel, dim3(static_cast<uint32_t>(n_blocks)), dim3(kCountThreads), 0, stream, a, counts, block_offsets);
   MFSDP_CHECK_LAUNCH("segment_tile_count_kernel");
+  const uint64_t bound = static_cast<uint64_t>(a.n_segments) * max_tiles_per_segment(a);
   hipLaunchKernelGGL(block_offset_kernel, dim3(1), dim3(kWave), 0, stream, block_offsets, n_blocks);
   MFSDP_CHECK_LAUNCH("block_offset_kernel");
-  const uint64_t bound = static_cast<uint64_t>(a.n_segments) * max_tiles_per_segment(a);
   // one tile per wave while the grid can hold them all (excess waves leave at once; beyond that the waves stride on)
   const uint64_t want = (bound + kChunkTiles * kWavesPerBlock - 1) / (kChunkTiles * kWavesPerBlock);
   const uint64_t cap = static_cast<uint64_t>(device_cu_count()) * kBalancedBlocksPerCu;
@@ -416,9 +421,8 @@ extern "C" int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_
   // tiles of the longest segment when its addresses allow 16-byte vectors (one more vector for a misaligned start)
   const uint64_t per_segment = (static_cast<uint64_t>(a.limit) * elem_bytes / 16 + kTileVectors) / kTileVectors;
   const uint64_t n_slots = static_cast<uint64_t>(n_segments) * per_segment;
-  const uint64_t want = (n_slots + kWavesPerBlock - 1) / kWavesPerBlock;
-  const dim3 grid(static_cast<uint32_t>(std::min<uint64_t>(want, (uint64_t{1} << 31) - 1)));
-  hipLaunchKernelGGL(segment_copy_uniform_kernel, grid, dim3(kCopyThreads), 0, as_stream(stream), a, per_segment, n_slots);
+  const dim3 grid(static_cast<uint32_t>(std::min<uint64_t>(n_slots, (uint64_t{1} << 31) - 1)));
+  hipLaunchKernelGGL(segment_copy_uniform_kernel, grid, dim3(kWave), 0, as_stream(stream), a, per_segment, n_slots);
   MFSDP_CHECK_LAUNCH("segment_copy_uniform_kernel");
   return MFSDP_OK;
 }
