@@ -106,7 +106,9 @@ int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_t local_num
  * library runs on holds its own copy until the process ends) instead of a caller's workspace, so the call neither
  * allocates nor frees anything; more than MFSDP_NOALLOC_MAX_SEGMENTS segments are rejected with
  * MFSDP_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (two
- * streams) race and must use mfsdp_copy_rank_segments_to_full_device with their own workspaces instead.
+ * streams) race and must use mfsdp_copy_rank_segments_to_full_device with their own workspaces instead.  The first
+ * call on a device looks the array's address up (and loads the code object it lives in): make it outside a graph
+ * capture; from the second call on the entry point only enqueues kernels.
  */
 #define MFSDP_NOALLOC_MAX_SEGMENTS 131071
 int mfsdp_copy_rank_segments_to_full_noalloc(const void* local, int64_t local_numel, void* output, int64_t output_numel,

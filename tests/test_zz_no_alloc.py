@@ -82,3 +82,36 @@ def test_more_segments_than_the_static_scratch_holds_are_rejected():
     _lib.check(call("mfsdp_copy_rank_segments_to_full_noalloc", local, out, meta, n_seg - 1, 4))
     torch.cuda.synchronize()
     assert out.tolist() == [1.0] * 8
+
+
+def test_replays_under_graph_capture_after_a_first_call_outside_it():
+    """The callers this entry point is for capture it into a HIP graph.  Its first call on a device looks the static
+    array's address up (and loads the code object), which belongs outside a capture; from the second call on it only
+    enqueues kernels.  Every replay is checked against the workspace entry point run eagerly, with the program's own
+    eager work and synchronisations between the replays."""
+    rng = np.random.default_rng(33)
+    torch.cuda.set_device(DEV)
+    n_seg, max_len = 300, 500
+    gs, ls, ln, local_n, out_n = layout(rng, n_seg, max_len)
+    meta = [torch.tensor(v, dtype=torch.int64, device=DEV) for v in (gs, ls, ln)]
+    ws = torch.empty(int(_lib.lib().mfsdp_copy_rank_segments_workspace_bytes(n_seg)), dtype=torch.uint8, device=DEV)
+    local = torch.zeros(local_n, dtype=torch.bfloat16, device=DEV)
+    have = torch.zeros(out_n, dtype=torch.bfloat16, device=DEV)
+    _lib.check(call("mfsdp_copy_rank_segments_to_full_noalloc", local, have, meta, n_seg, max(ln)))  # outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(call("mfsdp_copy_rank_segments_to_full_noalloc", local, have, meta, n_seg, max(ln)))
+    for seed in (1, 2, 3):
+        gen = torch.Generator().manual_seed(seed)
+        local.copy_(torch.randn(local_n, generator=gen).bfloat16())
+        base = torch.randn(out_n, generator=gen).bfloat16().to(DEV)
+        have.copy_(base)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = base.clone()
+        _lib.check(call("mfsdp_copy_rank_segments_to_full_device", local, want, meta, n_seg, max(ln), ws.data_ptr(), ws.numel()))
+        torch.cuda.synchronize()
+        assert not torch.equal(have, base)
+        assert torch.equal(have.view(torch.int16), want.view(torch.int16))
+        (local.float() * 2).sum().item()
