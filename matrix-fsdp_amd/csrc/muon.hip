@@ -65,8 +65,16 @@ bool plan_workspace(int64_t rows, int64_t cols, void* base, Workspace* w) {
 
 // Newton-Schulz on the update already sitting in w.xraw (rows x cols bf16) with per-block sums of squares in
 // w.partials.  Leaves O in param layout at *ortho with leading dimension *ldo.
+// The parameter update of the step, handed to the last product (see GemmNtArgs::update_param).
+struct ParamUpdate {
+  void* param = nullptr;
+  int dtype = MFSDP_F32;
+  float decay = 1.0f, neg_lr = 0.0f;
+};
+
+// With `update` and at least one step the last product writes the parameter itself and *ortho stays null.
 int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, float a, float b, float c, int steps,
-                      float eps, bool shared, const uint16_t** ortho, int* ldo, hipStream_t stream) {
+                      float eps, bool shared, const ParamUpdate* update, const uint16_t** ortho, int* ldo, hipStream_t stream) {
   if (int rc = muon_norm(w.partials, n_partials, eps, w.scalars, stream)) return rc;
   // the input is rows x cols; the iteration wants the short side first
   uint16_t* same = w.tall ? w.XT[0] : w.X[0];   // rows_pad x cols_pad
@@ -104,11 +112,20 @@ int run_newton_schulz(const Workspace& w, int rows, int cols, int n_partials, fl
     if (s + 1 == steps) {  // the last step only has to leave O in the parameter's orientation
       if (w.tall) g.skip_c = 1;
       else g.CT = nullptr;
+      if (update != nullptr) {  // ... or take it straight into the parameter: O is never stored
+        g.update_param = update->param;
+        g.update_dtype = update->dtype;
+        g.update_rows = rows;
+        g.update_cols = cols;
+        g.update_transposed = w.tall ? 1 : 0;
+        g.update_decay = update->decay;
+        g.update_neg_lr = update->neg_lr;
+      }
     }
     if (int rc = gemm_nt_bf16(g, w.gemm, stream)) return rc;
   }
   const int fin = steps & 1;
-  *ortho = w.tall ? w.XT[fin] : w.X[fin];
+  *ortho = (update != nullptr && steps > 0) ? nullptr : (w.tall ? w.XT[fin] : w.X[fin]);
   *ldo = w.tall ? w.mp : w.np;
   return MFSDP_OK;
 }
@@ -160,7 +177,7 @@ extern "C" int mfsdp_newton_schulz(const void* update, int update_dtype, int64_t
   if (int rc = muon_momentum(update, nullptr, update_dtype, rows * cols, 0.0, 0, false, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
-  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, false, &ortho, &ldo, s)) return rc;
+  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps, false, nullptr, &ortho, &ldo, s)) return rc;
   return muon_extract(out_bf16, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, s);
 }
 
@@ -180,13 +197,18 @@ extern "C" int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_
   if (int rc = muon_momentum(grad, momentum_buf, dtype, rows * cols, momentum, nesterov, true, w.xraw, w.partials, &n_partials, s)) return rc;
   const uint16_t* ortho = nullptr;
   int ldo = 0;
-  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps,
-                                 (flags & MFSDP_MUON_SHARED_MACHINE) != 0, &ortho, &ldo, s))
-    return rc;
   // the host scalars are doubles, as in Python: 1 - lr * wd and -adjusted_lr are rounded to fp32 once, where the
   // tensor operation takes them
-  const float decay = static_cast<float>(1.0 - lr * weight_decay);
-  return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, decay, static_cast<float>(-adjusted_lr), s);
+  ParamUpdate update;
+  update.param = param;
+  update.dtype = dtype;
+  update.decay = static_cast<float>(1.0 - lr * weight_decay);
+  update.neg_lr = static_cast<float>(-adjusted_lr);
+  if (int rc = run_newton_schulz(w, static_cast<int>(rows), static_cast<int>(cols), n_partials, a, b, c, steps, eps,
+                                 (flags & MFSDP_MUON_SHARED_MACHINE) != 0, &update, &ortho, &ldo, s))
+    return rc;
+  if (ortho == nullptr) return MFSDP_OK;  // the last product has updated the parameter
+  return muon_apply(param, dtype, ortho, static_cast<int>(rows), static_cast<int>(cols), ldo, update.decay, update.neg_lr, s);
 }
 
 extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf, int dtype, int64_t rows, int64_t cols, double lr,

@@ -27,6 +27,17 @@ struct GemmNtArgs {
   int d_transposed_is_q;  // the caller's word that Q holds D^T (Q[n][k] == D[k][n] for k < M): required with D, whose
                           // values whole tiles pick out of the Q slabs on their way through LDS (the fix-up of K-split
                           // pieces reads D itself)
+  // Parameter update in the epilogue (the last product of a Muon step): when update_param is set, nothing is stored to
+  // C / CT; every element o = bf16(alpha P Q^T + beta D) of the update_rows x update_cols corner instead goes into
+  //     param <- round(param * update_decay) + update_neg_lr * o        (torch/optim/_muon.py:313-315)
+  // on the contiguous row-major parameter of dtype update_dtype (MFSDP_F32 / MFSDP_BF16).  update_transposed: the
+  // parameter holds the transpose of C (update_rows counts C's columns then).  General products only.
+  void* update_param;
+  int update_dtype;
+  int update_rows, update_cols;
+  int update_transposed;
+  float update_decay, update_neg_lr;
+  int update_vectors;  // set by gemm_nt_bf16: groups of eight parameter elements may use 16-byte accesses
   int shared;  // other matrices' products run beside this one on other streams: a symmetric product then takes the
                // 256 x 256 tiles even where their triangle fills only part of the CUs (the rest works for the others)
 };

@@ -44,6 +44,52 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
+// param[prow][pcol .. pcol + count - 1] <- round(param * decay) + neg_lr * o for the first `count` bf16 values o of `eight`
+// (those inside the parameter's update_rows x update_cols); a.update_vectors says that whole groups of eight may use
+// 16-byte accesses.
+__device__ __forceinline__ void update_param8(const GemmNtArgs& a, int prow, int pcol, const u32x4& eight, int count = 8) {
+  if (prow >= a.update_rows || pcol >= a.update_cols) return;
+  const int n = a.update_cols - pcol < count ? a.update_cols - pcol : count;
+  const int64_t at = static_cast<int64_t>(prow) * a.update_cols + pcol;
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    o[2 * e] = __uint_as_float(eight[e] << 16);
+    o[2 * e + 1] = __uint_as_float(eight[e] & 0xffff0000u);
+  }
+  const float decay = a.update_decay, neg_lr = a.update_neg_lr;
+  if (a.update_dtype == MFSDP_F32) {
+    float* p = static_cast<float*>(a.update_param) + at;
+    if (n == 8 && a.update_vectors) {
+      f32x4 lo = reinterpret_cast<const f32x4*>(p)[0], hi = reinterpret_cast<const f32x4*>(p)[1];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = lo[e] * decay + neg_lr * o[e];
+        hi[e] = hi[e] * decay + neg_lr * o[4 + e];
+      }
+      reinterpret_cast<f32x4*>(p)[0] = lo;
+      reinterpret_cast<f32x4*>(p)[1] = hi;
+    } else {
+      for (int e = 0; e < n; ++e) p[e] = p[e] * decay + neg_lr * o[e];
+    }
+  } else {
+    uint16_t* p = static_cast<uint16_t*>(a.update_param) + at;
+    auto one = [&](uint16_t old, float ov) {
+      const float scaled = bf16_bits_to_float(__builtin_bit_cast(uint16_t, static_cast<__bf16>(bf16_bits_to_float(old) * decay)));
+      return __builtin_bit_cast(uint16_t, static_cast<__bf16>(scaled + neg_lr * ov));
+    };
+    if (n == 8 && a.update_vectors) {
+      u32x4 v = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        v[e] = static_cast<uint32_t>(one(static_cast<uint16_t>(v[e]), o[2 * e])) | (static_cast<uint32_t>(one(static_cast<uint16_t>(v[e] >> 16), o[2 * e + 1])) << 16);
+      *reinterpret_cast<u32x4*>(p) = v;
+    } else {
+      for (int e = 0; e < n; ++e) p[e] = one(p[e], o[e]);
+    }
+  }
+}
+
 struct Schedule {
   int tiles_m, tiles_n;
   int full_tiles;   // tiles computed whole, one per workgroup (block ids [0, full_tiles))
@@ -449,6 +495,37 @@ gemm_nt_kernel(GemmNtArgs a, Schedule sched) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[i][j][r] = a.alpha * acc[i][j][r];
+  if (a.update_param != nullptr) {
+    // the last product of a Muon step: the tile goes into the parameter (in the parameter's orientation) and nowhere else
+    if (!a.update_transposed) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            stage_c[(lrow + i * 16 + r) * kLdS + lcol + j * 16] = __builtin_bit_cast(uint16_t, static_cast<__bf16>(acc[i][j][r]));
+      __syncthreads();
+      for (int c = tid; c < BM * kRowChunks; c += kThreads) {
+        const int r = c / kRowChunks, cc = c - r * kRowChunks;
+        update_param8(a, row0 + r, col0 + cc * 8, *reinterpret_cast<const u32x4*>(stage_c + r * kLdS + cc * 8));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          u32x2 four = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
+          *reinterpret_cast<u32x2*>(stage_c + (lcol + j * 16) * kLdT + lrow + i * 16) = four;
+        }
+      __syncthreads();
+      for (int c = tid; c < BN * kColChunks; c += kThreads) {
+        const int r = c / kColChunks, cc = c - r * kColChunks;
+        update_param8(a, col0 + r, row0 + cc * 8, *reinterpret_cast<const u32x4*>(stage_c + r * kLdT + cc * 8));
+      }
+    }
+    return;
+  }
   if (!a.skip_c) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -533,6 +610,23 @@ splitk_fixup_kernel(GemmNtArgs a, Schedule sched) {
   }
   const uint32_t lo = pack_bf16x2(v[0], v[1]);
   const uint32_t hi = pack_bf16x2(v[2], v[3]);
+  if (a.update_param != nullptr) {  // uniform over the grid: the parameter update in place of the stores (see gemm_nt_kernel)
+    if (!a.update_transposed) {
+      const u32x4 packed = {lo, hi, 0u, 0u};  // this thread's four columns
+      update_param8(a, row, col, packed, 4);
+      return;
+    }
+    transposed[c][r] = static_cast<uint16_t>(lo);
+    transposed[c + 1][r] = static_cast<uint16_t>(lo >> 16);
+    transposed[c + 2][r] = static_cast<uint16_t>(hi);
+    transposed[c + 3][r] = static_cast<uint16_t>(hi >> 16);
+    __syncthreads();
+    if (t < kSub * 8) {
+      const int tr = t / 8, chunk = t % 8;
+      update_param8(a, tn * BN + sub_col0 + tr, tm * BM + sub_row0 + chunk * 8, *reinterpret_cast<const u32x4*>(&transposed[tr][chunk * 8]));
+    }
+    return;
+  }
   if (!a.skip_c) {
     const u32x2 packed = {lo, hi};
     *reinterpret_cast<u32x2*>(C + static_cast<int64_t>(row) * a.ldc + col) = packed;
@@ -679,7 +773,16 @@ int gemm_nt_bf16(const GemmNtArgs& a, const GemmScratch& scratch, hipStream_t st
   if (a.D && (!a.d_transposed_is_q || a.K < a.M || a.alpha == 0.0f))
     return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: a D operand needs D^T == Q (K >= M) and alpha != 0");
   if (a.ldp > (1 << 22) || a.ldq > (1 << 22)) return fail(MFSDP_ERR_UNSUPPORTED, "gemm_nt_bf16: leading dimensions beyond 2^22 elements");
-  const GemmNtArgs& b = a;
+  GemmNtArgs b = a;
+  if (a.update_param != nullptr) {
+    const int elem = a.update_dtype == MFSDP_F32 ? 4 : 2;
+    if (a.symmetric || (a.update_dtype != MFSDP_F32 && a.update_dtype != MFSDP_BF16) || a.update_rows <= 0 || a.update_cols <= 0 ||
+        a.update_rows > (a.update_transposed ? a.N : a.M) || a.update_cols > (a.update_transposed ? a.M : a.N) ||
+        reinterpret_cast<uintptr_t>(a.update_param) % elem)
+      return fail(MFSDP_ERR_INVALID, "gemm_nt_bf16: parameter update needs a general product, an f32 / bf16 parameter inside the result and an aligned pointer");
+    // groups of eight elements start at multiples of eight columns: whole 16-byte accesses when the rows keep that alignment
+    b.update_vectors = a.update_cols % 8 == 0 && reinterpret_cast<uintptr_t>(a.update_param) % 16 == 0;
+  }
   const GemmTuning tuning = tuning_snapshot();
   // Slabs of 32 (three to five deep) were measured too: each slab row is then half a 128-byte line, the vector
   // cache looks every line up twice, and the products run 15-25 % slower than with slabs of 64 two deep.
