@@ -34,7 +34,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 NS_COEFFS = (3.4445, -4.7750, 2.0315)
-# figures taken from the committed rocprofv3 counter profiles (they cannot be measured from inside this process)
+# Figures QUOTED from the committed rocprofv3 counter profiles (counters cannot be read from inside this process).  They
+# describe the library as it was when the profile was taken (its `head` line) and are reported under keys that say so.
 PROFILED_TRAFFIC = {"bytes_per_launch": 812_818_425, "source": "profiles/segment_program_hbm_traffic.md"}
 PROFILED_MUON = {
     # SQ_VALU_MFMA_BUSY_CYCLES over the SIMD cycles of the dispatch (all 256 CUs), per kernel and launch shape
@@ -59,8 +60,13 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=0, help="layer buffers of the hidden4096 workload (0 = all 32)")
     ap.add_argument("--skip-legs", action="store_true", help="only the timed pack/unpack region (used under rocprofv3)")
     ap.add_argument("--skip-mixed", action="store_true", help="skip the hidden5120 mixed-step leg")
-    ap.add_argument("--legs", default="ceiling,rows,muon,adamw,mixed",
-                    help="comma list of the extra legs to run: ceiling (plain copy / read-only / write-only probes), rows (hidden2048 row split), muon, adamw, mixed")
+    ap.add_argument("--legs", default="ceiling,rows,devcopy,gemm,muon,adamw,mixed",
+                    help="comma list of the extra legs to run: ceiling (plain copy / read-only / write-only probes), rows (hidden2048 row split), "
+                    "devcopy (the device-metadata rank-segment copy, the reference extension's own entry point), gemm (one plain 8192^3 product beside "
+                    "the library's), muon, adamw, mixed")
+    ap.add_argument("--muon-form", default="both", choices=("both", "serial", "side-by-side"),
+                    help="which form of the Muon leg to run: one matrix at a time on the calling stream, the three side by side on side streams, "
+                    "or both (serial alone makes every kernel of a rocprofv3 trace run by itself)")
     ap.add_argument("--skip-cpu", action="store_true", help="do not time the CPU baselines")
     ap.add_argument("--hold-muon-seconds", type=float, default=0.0,
                     help="after the Muon leg, keep stepping for this long (for sampling the clock beside it); reports the rate of that stretch")
@@ -188,7 +194,7 @@ def main() -> int:
         # HBM bytes per launch: not measurable from inside the run; the figure of the committed counter profile of this
         # workload (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a plain 1 GiB copy), quoted only for the run it describes
         "traffic": PROFILED_TRAFFIC["bytes_per_launch"] if layers == w.layers else None,
-        "traffic_source": PROFILED_TRAFFIC["source"] if layers == w.layers else None,
+        "traffic_source": (PROFILED_TRAFFIC["source"] + " (quoted, not measured by this run)") if layers == w.layers else None,
         "algorithmic_bytes_per_launch": bytes_per_launch,
         "avg_launch_ms": round(avg_launch_ms, 5),
         "launches_timed": len(launch_events) * 2 * layers,
@@ -321,6 +327,88 @@ def main() -> int:
         del full2, gath2, out2, grads2, packed32
         torch.cuda.empty_cache()
 
+    if "devcopy" in want:
+        # -------------------------------------------------------------- the boundary function itself: copy_rank_segments_to_full with
+        # DEVICE metadata (kernels/native/matrix_copy.cpp:53-83), one rank's shard of one hidden4096 layer buffer into the full buffer
+        import ctypes
+
+        from matrix_fsdp_amd.kernels import native as N
+        from matrix_fsdp_amd.kernels.segment_program import local_segments_program
+
+        segs = plan.rank_segments[0]
+        local = torch.empty(plan.shard_sizes[0], dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02)
+        out_full = torch.zeros(plan.total_numel, dtype=torch.bfloat16, device=dev)
+        gs, ls, ln, mx = N._segment_metadata_tensors(tuple(segs), device=dev)
+        ws_dc = N.copy_rank_segments_workspace(len(segs), dev)
+        moved = 2 * 2 * sum(sg.numel for sg in segs)  # bytes read + bytes written
+        stream = torch.cuda.current_stream(dev).cuda_stream
+
+        def noalloc():
+            _lib.check(_lib.lib().mfsdp_copy_rank_segments_to_full_noalloc(
+                local.data_ptr(), local.numel(), out_full.data_ptr(), out_full.numel(), gs.data_ptr(), ls.data_ptr(), ln.data_ptr(),
+                len(segs), int(mx), 2, stream))
+
+        prog_dc = local_segments_program(segs, local.numel(), plan.total_numel, torch.bfloat16, device=dev)
+        leg = {"segments": len(segs), "bytes_moved": moved}
+        for name, fn in (
+            ("uniform_launch_shape", lambda: N.copy_rank_segments_to_full(local, out_full, gs, ls, ln, mx)),
+            ("balanced_launch_shape", lambda: N.copy_rank_segments_to_full(local, out_full, gs, ls, ln, mx, workspace=ws_dc)),
+            ("noalloc_entry_point", noalloc),
+            ("compiled_segment_program_same_copy", lambda: prog_dc.run((local,), out_full)),
+        ):
+            med, _ = time_launches(torch, fn, 30, 5)
+            leg[name] = {"us": round(med * 1e3, 2), "GBps": round(moved / (med * 1e-3) / 1e9, 1), "pct_hbm_peak": round(100 * moved / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        want_full = torch.zeros_like(out_full)
+        prog_dc.run((local,), want_full)
+        assert torch.equal(out_full, want_full)
+        leg["note"] = ("mfsdp_copy_rank_segments_to_full_device on rank 0's shard of one hidden4096 layer buffer (row segments of a 2x2 block shard), "
+                       "metadata in device memory; uniform = one tile slot per (segment, tile index), balanced = byte-balanced grid behind two count kernels "
+                       "(for layouts whose segment lengths differ widely), noalloc = balanced with the library's static scratch")
+        legs["device_metadata_copy"] = leg
+        del local, out_full, ws_dc, want_full, prog_dc
+        torch.cuda.empty_cache()
+
+    if "gemm" in want:
+        # -------------------------------------------------------------- one plain product through the Newton-Schulz kernel beside
+        # the library's kernel for the same product (what torch.optim.Muon runs on)
+        n_g = 8192
+        pg = torch.empty(n_g, n_g, dtype=torch.bfloat16, device=dev).normal_()
+        qg = torch.empty(n_g, n_g, dtype=torch.bfloat16, device=dev).normal_()
+        cg = torch.empty(n_g, n_g, dtype=torch.bfloat16, device=dev)
+        scratch_g = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+
+        def ours():
+            _lib.check(_lib.lib().mfsdp_gemm_nt_bf16(pg.data_ptr(), qg.data_ptr(), cg.data_ptr(), n_g, n_g, n_g, scratch_g.data_ptr(), scratch_g.numel(), stream))
+
+        def library():
+            torch.matmul(pg, qg.T, out=cg)
+
+        fl = 2.0 * n_g**3
+        leg = {"shape": f"{n_g} x {n_g} x {n_g}, C = P Q^T, bf16, fp32 accumulation"}
+        for name, fn in (("gemm_nt_kernel", ours), ("library_torch_matmul", library)):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t0 < 1.0:  # long enough for the clock to settle at its sustained level
+                for _ in range(20):
+                    fn()
+                torch.cuda.synchronize()
+                reps += 20
+            sustained = (time.perf_counter() - t0) / reps
+            med, _ = time_launches(torch, fn, 20, 2)
+            leg[name] = {"us": round(med * 1e3, 1), "TFLOPs": round(fl / (med * 1e-3) / 1e12, 1),
+                         "sustained_TFLOPs_over_1s": round(fl / sustained / 1e12, 1), "pct_bf16_mfma_peak": round(100 * fl / (med * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 2)}
+        ours()
+        torch.cuda.synchronize()
+        check = torch.matmul(pg[:256].float(), qg[:256].float().T)
+        assert torch.allclose(cg[:256, :256].float(), check, rtol=2e-2, atol=2.0)
+        legs["gemm_8192_cubed"] = leg
+        del pg, qg, cg, scratch_g
+        torch.cuda.empty_cache()
+
     if "muon" in want:
         # -------------------------------------------------------------- Muon on the hidden4096 matrices
         ws = F.MuonWorkspace(dev)
@@ -341,20 +429,29 @@ def main() -> int:
             # the step of the optimizer: independent matrices side by side on the library's side streams, joined on this stream
             F.muon_step_many([(p, g, buf, kw) for p, g, buf in mats])
 
-        med_one_stream, _ = time_launches(torch, muon_one_by_one, 20, 5)
-        med, _ = time_launches(torch, muon_all, 20, 5)
+        med_one_stream = med = None
+        if args.muon_form in ("both", "serial"):
+            med_one_stream, _ = time_launches(torch, muon_one_by_one, 20, 5)
+        if args.muon_form in ("both", "side-by-side"):
+            med, _ = time_launches(torch, muon_all, 20, 5)
+        if med is None:
+            med = med_one_stream  # the step's time in the one form that was run
         flops = 0
         per_matrix = {}
         for (p, g, buf), shape in zip(mats, MUON_HIDDEN4096_SHAPES):
             m, n = min(shape), max(shape)
             fl = 5 * (4 * m * m * n + 2 * m**3)
             flops += fl
+            if args.muon_form == "side-by-side":
+                continue
             t, _ = time_launches(torch, lambda: F.muon_step(p, g, buf, workspace=ws, **kw), 20, 5)
-            per_matrix[f"{shape[0]}x{shape[1]}"] = {"ms": round(t, 4), "TFLOPs": round(fl / (t * 1e-3) / 1e12, 1)}
+            fl_exec = int(_lib.lib().mfsdp_muon_executed_flops(shape[0], shape[1], 5, 0))
+            per_matrix[f"{shape[0]}x{shape[1]}"] = {"ms": round(t, 4), "TFLOPs_executed": round(fl_exec / (t * 1e-3) / 1e12, 1),
+                                                    "TFLOPs_reference_flop_count": round(fl / (t * 1e-3) / 1e12, 1)}
         # the optimizer the reference builds for these parameters (torch.optim.Muon: hipBLASLt products, full GEMMs), same
         # GPU, same hyper-parameters, on copies of the tensors: the reference's own execution of this step, for scale
         torch_ms = None
-        if hasattr(torch.optim, "Muon"):
+        if hasattr(torch.optim, "Muon") and args.muon_form == "both":
             t_params = [torch.nn.Parameter(p.clone()) for p, _, _ in mats]
             t_opt = torch.optim.Muon(t_params, lr=kw["lr"], weight_decay=kw["weight_decay"], momentum=kw["momentum"], nesterov=kw["nesterov"],
                                      ns_coefficients=NS_COEFFS, eps=kw["eps"], ns_steps=kw["ns_steps"])
@@ -365,7 +462,8 @@ def main() -> int:
         tflops = flops / (med * 1e-3) / 1e12
         legs["muon_hidden4096"] = {
             "ms_per_step": round(med, 4),
-            "ms_per_step_one_matrix_at_a_time": round(med_one_stream, 4),
+            "form_timed": {"both": "side by side (muon_step_many)", "serial": "one matrix at a time", "side-by-side": "side by side (muon_step_many)"}[args.muon_form],
+            "ms_per_step_one_matrix_at_a_time": None if med_one_stream is None else round(med_one_stream, 4),
             "ns_TFLOPs_reference_flop_count": round(tflops, 1),
             "pct_bf16_mfma_peak": round(100 * tflops / BF16_MFMA_PEAK_TFLOPS, 2),
             "flop_count": "5 * (4 m^2 n + 2 m^3) per matrix, full GEMMs as the reference executes them; the time is the whole "
@@ -387,7 +485,7 @@ def main() -> int:
                 n_hold += 20
             held = (time.perf_counter() - t_hold) / n_hold * 1e3
             legs["muon_hidden4096"]["held"] = {"seconds": args.hold_muon_seconds, "ms_per_step": round(held, 4), "ns_TFLOPs_reference_flop_count": round(flops / (held * 1e-3) / 1e12, 1)}
-        executed = sum(int(_lib.lib().mfsdp_muon_executed_flops(sh[0], sh[1], 5, _lib.MUON_SHARED_MACHINE)) for sh in MUON_HIDDEN4096_SHAPES)
+        executed = sum(int(_lib.lib().mfsdp_muon_executed_flops(sh[0], sh[1], 5, 0 if args.muon_form == "serial" else _lib.MUON_SHARED_MACHINE)) for sh in MUON_HIDDEN4096_SHAPES)
         tflops_executed = executed / (med * 1e-3) / 1e12
         legs["muon_hidden4096"]["ns_TFLOPs_executed"] = round(tflops_executed, 1)
         result["roofline_muon"] = {
@@ -403,10 +501,9 @@ def main() -> int:
             "achieved_executed": round(tflops_executed, 1),
             "frac_executed": round(tflops_executed / BF16_MFMA_PEAK_TFLOPS, 4),
             "executed_over_reference_flops": round(executed / flops, 4),
-            # counter figures of the committed profiles of this leg (they cannot be measured from inside this process)
-            "mfma_busy": PROFILED_MUON["mfma_busy"],
-            "traffic": PROFILED_MUON["traffic_bytes_per_launch"],
-            "traffic_source": PROFILED_MUON["source"],
+            # counter figures QUOTED from the committed profiles of this leg (not measured by this run; see their `head` lines)
+            "quoted_from_profiles": {"mfma_busy": PROFILED_MUON["mfma_busy"], "traffic_bytes_dominant_launch": PROFILED_MUON["traffic_bytes_per_launch"],
+                                     "source": PROFILED_MUON["source"]},
         }
         del mats
         torch.cuda.empty_cache()

@@ -196,21 +196,6 @@ int mfsdp_segment_program_run(mfsdp_segment_program* program, const void* const*
 int mfsdp_segment_program_run_many(mfsdp_segment_program* program, int32_t n_buffers, const void* const* srcs,
                                    int32_t n_srcs, void* const* dsts, void* stream);
 
-/* Launch tuning for experiments (safe to call while other threads launch): workgroups per CU of the copy grid
- * (-1 = library default, 0 = one workgroup per four tiles without a grid-stride loop, n > 0 = persistent grid of n
- * per CU), non-temporal hints (0 none, 1 loads and stores, 2 loads only, 3 stores only, -1 = default); and, for
- * programs created afterwards, 128-bit loads in flight per lane (1, 2 or 4; 0 = default); threads per workgroup (64, 128
- * or 256: the 256 lanes of a tile spread over 4, 2 or 1 workgroups; 0 = default). */
-void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll, int block_threads);
-
-/*
- * Measurement aid (no counterpart in the reference): one pass of pure reads (kind 0: `bytes` of src are loaded
- * and discarded; dst is a 4 KiB sink that is never written as long as src holds no all-ones 16-byte group) or pure
- * writes (kind 1: `bytes` of dst are filled with a constant), one workgroup per 4 KiB like the copy kernels, so that a
- * benchmark can state what the part sustains in each direction beside the copy it measures.
- */
-int mfsdp_hbm_probe(int kind, const void* src, void* dst, int64_t bytes, void* stream);
-
 /* ------------------------------------------------------------------ cast */
 
 /*
@@ -235,13 +220,6 @@ int mfsdp_accumulate(void* dst, const void* src, int64_t numel, int dtype, void*
  * rows x cols matrix (0 on invalid shape).
  */
 int64_t mfsdp_muon_workspace_bytes(int64_t rows, int64_t cols);
-
-/*
- * Flops the Newton-Schulz kernels execute for `steps` iterations on a rows x cols matrix with the current tuning
- * and the flags of mfsdp_muon_step_ex (operands zero-padded to multiples of 256; the two symmetric products of a step compute only the tiles on or below
- * the diagonal).  The reference executes full products: steps * (4 m^2 n + 2 m^3) with m the short side.
- */
-int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps, int flags);
 
 /*
  * Quintic Newton-Schulz orthogonalisation of one matrix, the arithmetic of
@@ -282,13 +260,6 @@ int mfsdp_muon_step_ex(void* param, const void* grad, void* momentum_buf, int dt
                        float a, float b, float c, int steps, float eps, double adjusted_lr, int flags,
                        void* workspace, int64_t workspace_bytes, void* stream);
 
-/* Kernel selection for experiments (values <= 0 keep the current setting):
- * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
- * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU; for the symmetric products also 3, the default:
- * whichever of the two fills the CUs better for the size at hand), the tile rows the general products walk together
- * (default 4), K-splitting of the last partial round of tiles on (1) / off (2), and its cap. */
-void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder, int max_splits);
-
 /* ------------------------------------------------------------------ AdamW */
 
 /*
@@ -315,6 +286,50 @@ int mfsdp_adamw_step(float* param, const void* grad, int grad_dtype, float* exp_
 int mfsdp_adamw_step_ex(float* param, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
                         float* max_exp_avg_sq, int64_t numel, int64_t step, double lr, double beta1, double beta2,
                         double eps, double weight_decay, int maximize, void* stream);
+
+/* ------------------------------------------------------------------ measurement and experiments
+ *
+ * Nothing below is part of the drop-in surface: the reference has no counterpart for any of it and a binding of the
+ * reference needs none of it.  bench.py and the tests use these entry points to state what the part sustains beside
+ * what the kernels reach, to count the flops the kernels execute, and to force kernel variants.
+ */
+
+/*
+ * Flops the Newton-Schulz kernels execute for `steps` iterations on a rows x cols matrix with the current tuning
+ * and the flags of mfsdp_muon_step_ex (operands zero-padded to multiples of 256; the two symmetric products of a step compute only the tiles on or below
+ * the diagonal).  The reference executes full products: steps * (4 m^2 n + 2 m^3) with m the short side.
+ */
+int64_t mfsdp_muon_executed_flops(int64_t rows, int64_t cols, int steps, int flags);
+
+/*
+ * Measurement aid (no counterpart in the reference): one pass of pure reads (kind 0: `bytes` of src are loaded
+ * and discarded; dst is a 4 KiB sink that is never written as long as src holds no all-ones 16-byte group) or pure
+ * writes (kind 1: `bytes` of dst are filled with a constant), one workgroup per 4 KiB like the copy kernels, so that a
+ * benchmark can state what the part sustains in each direction beside the copy it measures.
+ */
+int mfsdp_hbm_probe(int kind, const void* src, void* dst, int64_t bytes, void* stream);
+
+/*
+ * One plain product C = bf16(P Q^T) through the Newton-Schulz GEMM kernel (P: m x k, Q: n x k, C: m x n, all bf16
+ * row-major and contiguous, m and n multiples of 256, k of 64), so that a benchmark can time the kernel on a shape of
+ * its choice beside a library GEMM.  `partials` (may be NULL) is scratch for the K-split pieces of a last partial
+ * round of tiles.
+ */
+int mfsdp_gemm_nt_bf16(const void* p, const void* q, void* c, int m, int n, int k, void* partials, int64_t partials_bytes, void* stream);
+
+/* Launch tuning for experiments (safe to call while other threads launch): workgroups per CU of the copy grid
+ * (-1 = library default, 0 = one workgroup per four tiles without a grid-stride loop, n > 0 = persistent grid of n
+ * per CU), non-temporal hints (0 none, 1 loads and stores, 2 loads only, 3 stores only, -1 = default); and, for
+ * programs created afterwards, 128-bit loads in flight per lane (1, 2 or 4; 0 = default); threads per workgroup (64, 128
+ * or 256: the 256 lanes of a tile spread over 4, 2 or 1 workgroups; 0 = default). */
+void mfsdp_set_copy_tuning(int blocks_per_cu, int nontemporal, int unroll, int block_threads);
+
+/* Kernel selection for experiments (values <= 0 keep the current setting):
+ * tile variant of the general and of the symmetric Newton-Schulz products (1: 256x256 tile / 8 waves / one
+ * workgroup per CU, 2: 128x128 tile / 4 waves / two per CU; for the symmetric products also 3, the default:
+ * whichever of the two fills the CUs better for the size at hand), the tile rows the general products walk together
+ * (default 4), K-splitting of the last partial round of tiles on (1) / off (2), and its cap. */
+void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder, int max_splits);
 
 #ifdef __cplusplus
 }

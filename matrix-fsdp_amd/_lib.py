@@ -21,7 +21,7 @@ CONVERT_F32_TO_F16 = 4
 DT_F32 = 0
 DT_BF16 = 1
 DT_F16 = 2  # mfsdp_accumulate only
-ABI_VERSION = 5
+ABI_VERSION = 6
 MUON_SHARED_MACHINE = 1
 NOALLOC_MAX_SEGMENTS = 131071  # MFSDP_NOALLOC_MAX_SEGMENTS
 
@@ -89,6 +89,7 @@ SIGNATURES = {
          c_float, c_float, c_float, c_int, c_float, c_double, c_int, c_void_p, c_int64, c_void_p],
     ),
     "mfsdp_set_muon_tuning": (None, [c_int, c_int, c_int, c_int, c_int]),
+    "mfsdp_gemm_nt_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int64, c_void_p]),
     "mfsdp_accumulate": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mfsdp_adamw_step": (
         c_int,

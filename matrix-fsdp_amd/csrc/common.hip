@@ -32,4 +32,4 @@ int device_cu_count() {
 }  // namespace mfsdp
 
 extern "C" const char* mfsdp_last_error(void) { return mfsdp::g_last_error; }
-extern "C" int mfsdp_abi_version(void) { return 5; }
+extern "C" int mfsdp_abi_version(void) { return 6; }

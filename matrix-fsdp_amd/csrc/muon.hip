@@ -218,6 +218,18 @@ extern "C" int mfsdp_muon_step(void* param, const void* grad, void* momentum_buf
                             adjusted_lr, 0, workspace, workspace_bytes, stream);
 }
 
+extern "C" int mfsdp_gemm_nt_bf16(const void* p, const void* q, void* c, int m, int n, int k, void* partials, int64_t partials_bytes, void* stream) {
+  GemmNtArgs g{};
+  g.P = p; g.Q = q; g.C = c;
+  g.M = m; g.N = n; g.K = k;
+  g.ldp = k; g.ldq = k; g.ldc = n;
+  g.alpha = 1.0f;
+  GemmScratch scratch;
+  scratch.partials = partials;
+  scratch.partials_bytes = partials ? partials_bytes : 0;
+  return gemm_nt_bf16(g, scratch, as_stream(stream));
+}
+
 extern "C" void mfsdp_set_muon_tuning(int general_variant, int symmetric_variant, int group_m, int split_remainder,
                                       int max_splits) {
   GemmTuning t = get_gemm_tuning();
