@@ -26,6 +26,7 @@ constexpr int kMaxBatch = 64;     // destination pointers (buffers) one launch c
 constexpr int kDefaultBlocksPerCu = 0;  // one workgroup per tile
 constexpr int kDefaultBlockThreads = 64;
 constexpr int kBlockThreads = 256;
+constexpr int kFillTileSpans = 8;  // spans of 256 * U groups a zero-fill tile covers (its group count must stay below 2^16)
 constexpr int64_t kMaxGrid = (int64_t{1} << 31) - 1;  // grid-stride loops keep a capped grid correct
 constexpr int64_t kMaxUnitsPerRun = 0x7fffffff;  // a device run holds fewer than 2^31 units: the reciprocal division is exact below 2^31 groups, at any group width
 
@@ -385,8 +386,14 @@ int compile_tables(mfsdp_segment_program* prog, std::vector<Compiled>* out) {
     if (r.rows == 1 || row_groups >= tile_groups / 2) {
       // direct tiles: every row is cut into equal pieces of at most one tile, a multiple of 128 bytes long where
       // the row allows it, so that no workgroup is left with a sliver
-      const int64_t per_row = (row_groups + tile_groups - 1) / tile_groups;
-      const int64_t piece = std::min<int64_t>(tile_groups, ((row_groups + per_row - 1) / per_row + 7) / 8 * 8);
+      // Zero fill only stores: a wavefront that writes 1 KiB is gone before the next can be dispatched and the launch
+      // runs at the dispatch rate (pad tails of the hidden5120 owner layouts: 4.2-4.6 TB/s); eight times the span per
+      // workgroup, walked in the kernel's loop over a direct tile, lifts the fill to 5.3 TB/s (pack of such a layer
+      // buffer 6.09 TB/s against 5.55-5.78; 32 spans no better; fill tiles spread evenly among the copying tiles
+      // instead of behind each rank's segments: slower, 5.85-5.95).
+      const int64_t tile_cap = r.src_id < 0 ? kFillTileSpans * tile_groups : tile_groups;
+      const int64_t per_row = (row_groups + tile_cap - 1) / tile_cap;
+      const int64_t piece = std::min<int64_t>(tile_cap, ((row_groups + per_row - 1) / per_row + 7) / 8 * 8);
       for (int64_t row = 0; row < r.rows; ++row) {
         for (int64_t col = 0; col < row_groups; col += piece) {
           const uint64_t n = static_cast<uint64_t>(std::min(piece, row_groups - col));
