@@ -54,10 +54,12 @@ bool plan_workspace(int64_t rows, int64_t cols, void* base, Workspace* w) {
   w->XT[1] = reinterpret_cast<uint16_t*>(take(x_bytes));
   w->A = reinterpret_cast<uint16_t*>(take(a_bytes));
   w->B = reinterpret_cast<uint16_t*>(take(a_bytes));
-  w->partials = reinterpret_cast<float*>(take(round_up(kMuonMaxPartials * 4, kAlign)));
   w->scalars = reinterpret_cast<float*>(take(kAlign));
   w->gemm.partials = take(kGemmPartialsBytes);
   w->gemm.partials_bytes = kGemmPartialsBytes;
+  // the sums of squares of the momentum kernel are consumed by the norm before the first product runs
+  static_assert(kMuonMaxPartials * 4 <= kGemmPartialsBytes, "the partial sums borrow the products' scratch");
+  w->partials = reinterpret_cast<float*>(w->gemm.partials);
   w->xraw = w->X[1];
   w->bytes = off;
   return true;

@@ -7,7 +7,7 @@
 
 namespace mfsdp {
 
-constexpr int kMuonMaxPartials = 2048;
+constexpr int kMuonMaxPartials = 1 << 18;  // workgroups of the momentum kernel = partial sums of squares (1 MiB of fp32)
 
 // xraw <- bf16(u), partials <- per-block sums of bf16(u)^2, where u is the momentum/Nesterov update
 // (with_momentum; buf updated in place) or grad itself.  dtype: MFSDP_F32 / MFSDP_BF16 of grad and buf.
