@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -159,14 +160,35 @@ def _underfills_the_machine(shape, compute_units: int) -> bool:
     return 4 * (t * (t + 1) // 2) < 3 * compute_units
 
 
-def muon_step_many(jobs, *, workspace: MuonWorkspace | None = None, pool: MuonStreamPool | None = None) -> None:
+def side_by_side_default() -> bool | None:
+    """``MATRIX_FSDP_MUON_SIDE_BY_SIDE``: ``0`` keeps every matrix on the calling stream (result bits that do not
+    depend on which other parameters the optimizer holds), ``1`` forces the side streams, unset / ``auto`` decides
+    per call."""
+    value = os.environ.get("MATRIX_FSDP_MUON_SIDE_BY_SIDE", "auto").strip().lower()
+    if value in ("0", "false", "off", "no"):
+        return False
+    if value in ("1", "true", "on", "yes"):
+        return True
+    return None
+
+
+def muon_step_many(jobs, *, workspace: MuonWorkspace | None = None, pool: MuonStreamPool | None = None,
+                   side_by_side: bool | None = None) -> None:
     """Updates several matrices; ``jobs`` is a sequence of ``(param, grad, momentum_buf, keywords of muon_step)``.
 
     The matrices of a rank are independent of each other.  When at least two of them are so small that the triangle
-    of their symmetric products leaves CUs idle (a hidden4096 layer on 256 CUs: 136 tiles), they are spread over up to
-    three side streams, longest first, so that those CUs work for another matrix (three hidden4096 matrices: 7.97
-    against 8.47 ms); the calling stream waits for the side streams before anything enqueued later runs.  Otherwise
-    (larger matrices keep the machine busy on their own) they run one after the other on the calling stream."""
+    of their symmetric products leaves CUs idle (a hidden4096 layer on 256 CUs: 136 tiles), those are spread over up
+    to three side streams, longest first, so that the idle CUs work for another matrix (three hidden4096 matrices:
+    7.3 against 7.5 ms); the calling stream waits for the side streams before anything enqueued later runs.  Matrices
+    that keep the machine busy on their own run first, one after the other on the calling stream, as every matrix does
+    when fewer than two are small.
+
+    Reproducibility: a matrix updated on a side stream takes 256 x 256 tiles in its symmetric products where it would
+    take 128 x 128 tiles alone, so the order of its fp32 sums, and with it the last bits of the update, depends on
+    whether other small matrices are updated in the same call.  Both forms meet the same parity bar; a caller that
+    needs bits independent of the optimizer's other parameters passes ``side_by_side=False`` (or sets
+    ``MATRIX_FSDP_MUON_SIDE_BY_SIDE=0``), which keeps everything on the calling stream; ``True`` sends every 2-D
+    matrix to the side streams whatever its size."""
     jobs = list(jobs)
     if not jobs:
         return
@@ -174,12 +196,25 @@ def muon_step_many(jobs, *, workspace: MuonWorkspace | None = None, pool: MuonSt
     for param, *_ in jobs:
         if param.device != device:
             raise RuntimeError("muon_step_many updates the matrices of one device")
+    if side_by_side is None:
+        side_by_side = side_by_side_default()
     compute_units = torch.cuda.get_device_properties(device).multi_processor_count
-    small = sum(1 for param, *_ in jobs if param.ndim == 2 and _underfills_the_machine(param.shape, compute_units))
-    if small < 2:
+    if side_by_side is False:
+        small = []
+    elif side_by_side:
+        small = [job for job in jobs if job[0].ndim == 2]
+    else:
+        small = [job for job in jobs if job[0].ndim == 2 and _underfills_the_machine(job[0].shape, compute_units)]
+        if len(small) < 2:
+            small = []
+    small_ids = {id(job) for job in small}
+    alone = [job for job in jobs if id(job) not in small_ids]
+    if alone:
         workspace = workspace or MuonWorkspace(device)
-        for param, grad, buf, kw in jobs:
+        for param, grad, buf, kw in alone:
             muon_step(param, grad, buf, workspace=workspace, **kw)
+    jobs = small
+    if not jobs:
         return
     if pool is None:
         pool = _STREAM_POOLS.get(device)

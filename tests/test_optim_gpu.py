@@ -162,6 +162,39 @@ def test_muon_step_many_matches_one_matrix_at_a_time():
     assert torch.equal(many_p[0], one_p[0])
 
 
+def test_muon_step_many_side_by_side_switch(monkeypatch):
+    """Matrices large enough that the side-by-side form changes the tiling of their symmetric products (m = 3072: the
+    triangle of 256 x 256 tiles occupies 78 of the CUs): with ``side_by_side=False`` (argument or environment) every
+    matrix gets the bits of a call of its own, whatever else the batch holds; the side-by-side form stays within the
+    parity bar of the same result."""
+    shapes = [(3072, 3072), (3072, 3328), (3072, 3072)]
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    params = [make(sh, 400 + i, 0.02).to(DEV) for i, sh in enumerate(shapes)]
+    grads = [make(sh, 500 + i).bfloat16().float().to(DEV) for i, sh in enumerate(shapes)]
+    ws = F.MuonWorkspace(DEV)
+    alone_p, alone_b = [p.clone() for p in params], [torch.zeros_like(p) for p in params]
+    for i in range(len(shapes)):
+        F.muon_step(alone_p[i], grads[i], alone_b[i], workspace=ws, **kw)
+
+    def batch(**how):
+        ps, bs = [p.clone() for p in params], [torch.zeros_like(p) for p in params]
+        F.muon_step_many([(ps[i], grads[i], bs[i], kw) for i in range(len(shapes))], **how)
+        torch.cuda.synchronize()
+        return ps, bs
+
+    ps, bs = batch(side_by_side=False)
+    assert all(torch.equal(a, b) for a, b in zip(ps, alone_p)) and all(torch.equal(a, b) for a, b in zip(bs, alone_b))
+    monkeypatch.setenv("MATRIX_FSDP_MUON_SIDE_BY_SIDE", "0")
+    ps, bs = batch()
+    assert all(torch.equal(a, b) for a, b in zip(ps, alone_p))
+    monkeypatch.delenv("MATRIX_FSDP_MUON_SIDE_BY_SIDE")
+    for how in (dict(), dict(side_by_side=True)):
+        ps, bs = batch(**how)
+        for i in range(len(shapes)):
+            assert rel_fro((ps[i] - params[i]).cpu(), (alone_p[i] - params[i]).cpu()) < MUON_TOL
+            assert torch.equal(bs[i], alone_b[i])  # the momentum does not depend on the tiling
+
+
 def test_muon_argument_errors():
     p = torch.zeros(8, 8, device=DEV)
     with pytest.raises(ValueError, match="2D"):
