@@ -40,10 +40,10 @@ PROFILED_TRAFFIC = {"bytes_per_launch": 812_818_425, "source": "profiles/segment
 PROFILED_MUON = {
     # SQ_VALU_MFMA_BUSY_CYCLES over the SIMD cycles of the dispatch (all 256 CUs), per kernel and launch shape
     "mfma_busy": {
-        "gemm_nt_kernel<256,256> general product, 768 workgroups (12288x4096)": 0.572,
-        "gemm_nt_kernel<256,256> general product, 688 workgroups (11008x4096)": 0.513,
-        "gemm_nt_kernel<256,256> general product, 256 workgroups (4096x4096)": 0.600,
-        "gemm_nt_kernel<128,128> symmetric products, one matrix at a time, 768 workgroups": 0.476,
+        "gemm_nt_kernel<256,256> general product, 768 workgroups (12288x4096)": 0.565,
+        "gemm_nt_kernel<256,256> general product, 688 workgroups (11008x4096)": 0.508,
+        "gemm_nt_kernel<256,256> general product, 256 workgroups (4096x4096)": 0.597,
+        "gemm_nt_kernel<128,128> symmetric products, one matrix at a time, 768 workgroups": 0.470,
     },
     # the dominant launch, B X on 12288 x 4096 (768 workgroups): FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, in bytes
     "traffic_bytes_per_launch": (2 * 295_250 + 176_947) * 1024,
