@@ -75,6 +75,28 @@ def test_newton_schulz_other_polynomials(coefficients):
     assert rel_fro(p_dev.cpu() - p, p_ref - p) < MUON_TOL
 
 
+@pytest.mark.parametrize("shape", [(192, 320), (320, 192), (100, 36), (37, 101)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("steps", [0, 1])
+def test_muon_step_with_no_or_one_newton_schulz_step(shape, dtype, steps):
+    """Without a Newton-Schulz step there is no product whose epilogue could carry the parameter update (the separate
+    update kernel runs on the normalised update); with one step the only update product is also the last one.  Wide,
+    tall and unaligned shapes (tall parameters are updated from the transposed tile)."""
+    p = make(shape, 31, 0.02).to(dtype)
+    g, buf = make(shape, 32).to(dtype), make(shape, 33).to(dtype)
+    kw = dict(lr=0.02, weight_decay=0.1, momentum=0.95, nesterov=True)
+    p_dev, buf_dev = p.to(DEV), buf.to(DEV)
+    F.muon_step(p_dev, g.to(DEV), buf_dev, ns_steps=steps, **kw)
+    p_ref, buf_ref = p.clone(), buf.clone()
+    O.muon_step(p_ref, g, buf_ref, steps=steps, **kw)
+    tol = MUON_TOL if dtype == torch.float32 else 0.05  # a bf16 parameter moves in steps of its own last bit
+    assert rel_fro(p_dev.cpu().float() - p.float(), p_ref.float() - p.float()) < tol
+    if dtype == torch.float32:
+        assert torch.allclose(buf_dev.cpu(), buf_ref, rtol=1e-6, atol=1e-9)
+    else:
+        assert (buf_dev.cpu().view(torch.int16).int() - buf_ref.view(torch.int16).int()).abs().max() <= 1
+
+
 def test_non_finite_coefficients_are_refused_before_anything_runs():
     p, g, buf = make((64, 64), 21, 0.02).to(DEV), make((64, 64), 22).to(DEV), make((64, 64), 23).to(DEV)
     before = (p.clone(), buf.clone())
