@@ -28,7 +28,7 @@ namespace mfsdp {
 namespace {
 
 constexpr int kWave = 64;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = 4;  // loads in flight per lane = 1 KiB spans per tile; on 4.7 KiB row segments: 1 -> 65 us, 2 -> 45, 4 -> 36, 8 -> 48
 constexpr int kTileVectors = kWave * kUnroll;
 constexpr int kCopyThreads = 64;  // one wavefront per workgroup
 constexpr int kWavesPerBlock = kCopyThreads / kWave;
@@ -42,7 +42,7 @@ static_assert(kBlockSegments == 1 << kBlockShift, "block of segments");
 // four waves: (8 tiles, 16 waves per CU) 50 us, (4, 64) 48 us, (1, 256) 45 us, (1, 1024) 59 us; eight segments of 50 MB:
 // 163, 176, 148, 155 us.  Many short-lived waves beat few long-lived ones, as in the other copy kernels, until the empty
 // workgroups of the upper-bound grid cost more than they hide.  One wavefront per workgroup (dispatch in index order
-// sweeps neighbouring addresses) took the uniform shape from 5.4-5.7 to 5.8-6.0 TB/s on that shard, the level of the
+// sweeps neighbouring addresses) took the uniform shape from 5.4-5.7 to 5.6-5.8 TB/s on that shard, close to the
 // compiled segment program; the balanced shape stays at 46 us there (its two count kernels are 9 us of that, and a
 // ballot search over the running counts in place of the bisection was slower still: 87 us -- the set-up of a wave that
 // moves 4 KiB is what costs), so it is the shape for layouts whose segment lengths differ widely, not for this one.
