@@ -210,12 +210,23 @@ __device__ __forceinline__ void copy_tiles_any(const Geometry& g, uint64_t tile_
 // segment's addresses force a narrower vector).
 // One wavefront per workgroup: workgroups are dispatched in index order, so the waves in flight sweep neighbouring
 // addresses (as in the other copy kernels, small short-lived workgroups serve HBM best).
+// FAST: fewer than 2^31 slots, so the slot's segment comes from a multiply-high by a host-computed reciprocal
+// (slots_per_segment >= 2; magic == 0 says one slot per segment) instead of a 64-bit division in every workgroup.
+template <bool FAST>
 __global__ void __launch_bounds__(kWave)
-segment_copy_uniform_kernel(SegmentCopyArgs a, uint64_t slots_per_segment, uint64_t n_slots) {
+segment_copy_uniform_kernel(SegmentCopyArgs a, uint64_t slots_per_segment, uint64_t n_slots, uint32_t magic, uint32_t shift) {
   const uint32_t lane = threadIdx.x;
   for (uint64_t slot = blockIdx.x; slot < n_slots; slot += gridDim.x) {
-    const uint64_t s = slot / slots_per_segment;
-    const uint64_t first = slot - s * slots_per_segment;
+    uint64_t s, first;
+    if constexpr (FAST) {
+      const uint32_t slot32 = static_cast<uint32_t>(slot);
+      const uint32_t s32 = magic == 0 ? slot32 : (__umulhi(magic, slot32) >> shift);
+      s = s32;
+      first = slot32 - s32 * static_cast<uint32_t>(slots_per_segment);
+    } else {
+      s = slot / slots_per_segment;
+      first = slot - s * slots_per_segment;
+    }
     const Geometry g = segment_geometry(a, static_cast<int64_t>(s));
     for (uint64_t tile = first; tile < g.tiles; tile += slots_per_segment) copy_tiles_any(g, tile, tile + 1, lane);
   }
@@ -422,7 +433,19 @@ extern "C" int mfsdp_copy_rank_segments_to_full_device(const void* local, int64_
   const uint64_t per_segment = (static_cast<uint64_t>(a.limit) * elem_bytes / 16 + kTileVectors) / kTileVectors;
   const uint64_t n_slots = static_cast<uint64_t>(n_segments) * per_segment;
   const dim3 grid(static_cast<uint32_t>(std::min<uint64_t>(n_slots, (uint64_t{1} << 31) - 1)));
-  hipLaunchKernelGGL(segment_copy_uniform_kernel, grid, dim3(kWave), 0, as_stream(stream), a, per_segment, n_slots);
+  if (n_slots < (uint64_t{1} << 31)) {
+    // floor(slot / d) for slot < 2^31 as umulhi(magic, slot) >> shift, with the round-up reciprocal of d >= 2
+    uint32_t magic = 0, shift = 0;
+    if (per_segment >= 2) {
+      uint32_t l = 0;
+      while ((uint64_t{1} << l) < per_segment) ++l;  // ceil(log2 d) >= 1
+      magic = static_cast<uint32_t>((static_cast<unsigned __int128>(1) << (31 + l)) / per_segment + 1);
+      shift = l - 1;
+    }
+    hipLaunchKernelGGL(segment_copy_uniform_kernel<true>, grid, dim3(kWave), 0, as_stream(stream), a, per_segment, n_slots, magic, shift);
+  } else {
+    hipLaunchKernelGGL(segment_copy_uniform_kernel<false>, grid, dim3(kWave), 0, as_stream(stream), a, per_segment, n_slots, 0u, 0u);
+  }
   MFSDP_CHECK_LAUNCH("segment_copy_uniform_kernel");
   return MFSDP_OK;
 }
